@@ -1,0 +1,152 @@
+"""Pins the CPU oracle (oracle/diff_attn_oracle.py) without importing the reference.
+
+Each test is chosen so that a plausible restatement mistake (a dropped term, a wrong sign, a
+transposed operand, eps in the wrong place, the (1 - lambda_init) factor applied without
+rms_norm) fails at least one of them.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import brute_force
+from oracle import diff_attn_oracle as orc
+
+
+def rand_inputs(B, H, N, D, seed=0, dtype=torch.float64, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda d: (torch.randn(B, H, N, d, generator=g, dtype=torch.float32) * scale).to(dtype)
+    return mk(D), mk(D), mk(D), mk(D), mk(2 * D)
+
+
+def test_lambda_zero_is_sdpa():
+    q1, q2, k1, k2, v = rand_inputs(2, 3, 40, 16, seed=1)
+    y = orc.forward(q1, q2, k1, k2, v, 0.0, rms_norm=False, dtype=torch.float64)
+    ref = F.scaled_dot_product_attention(q1, k1, v)
+    assert torch.allclose(y, ref, atol=1e-12)
+    y = orc.forward(q1, q2, k1, k2, v, 0.0, lambda_init=0.3, rms_norm=True, dtype=torch.float64)
+    ref = 0.7 * F.rms_norm(ref, (32,), eps=1e-5)
+    assert torch.allclose(y, ref, atol=1e-12)
+
+
+def test_identical_streams():
+    q1, _, k1, _, v = rand_inputs(1, 2, 33, 8, seed=2)
+    ref = F.scaled_dot_product_attention(q1, k1, v)
+    y = orc.forward(q1, q1, k1, k1, v, 0.25, rms_norm=False, dtype=torch.float64)
+    assert torch.allclose(y, 0.75 * ref, atol=1e-12)
+    y = orc.forward(q1, q1, k1, k1, v, 1.0, lambda_init=0.8, rms_norm=True, dtype=torch.float64)
+    assert torch.count_nonzero(y) == 0
+
+
+def test_zero_keys_gives_mean_of_v():
+    q1, q2, k1, k2, v = rand_inputs(1, 2, 17, 8, seed=3)
+    y = orc.forward(q1, q2, 0 * k1, 0 * k2, v, 0.4, rms_norm=False, dtype=torch.float64)
+    ref = 0.6 * v.mean(dim=2, keepdim=True).expand_as(v)
+    assert torch.allclose(y, ref, atol=1e-12)
+
+
+def test_single_key():
+    q1, q2, k1, k2, v = rand_inputs(2, 2, 1, 4, seed=4)
+    y = orc.forward(q1, q2, k1, k2, v, -0.5, rms_norm=False, dtype=torch.float64)
+    assert torch.allclose(y, 1.5 * v, atol=1e-12)
+
+
+def test_rmsnorm_invariants():
+    q1, q2, k1, k2, v = rand_inputs(1, 2, 24, 8, seed=5)
+    lam, li = 0.5, 0.8
+    x = orc.forward(q1, q2, k1, k2, v, lam, lambda_init=li, rms_norm=False, dtype=torch.float64)
+    y = orc.forward(q1, q2, k1, k2, v, lam, lambda_init=li, rms_norm=True, dtype=torch.float64)
+    m = x.pow(2).mean(-1)
+    assert torch.allclose(y.pow(2).mean(-1), (1 - li) ** 2 * m / (m + 1e-5), rtol=1e-10)
+    # without rms_norm there is no (1 - lambda_init) factor (src/layers.py:74-78)
+    x2 = orc.forward(q1, q2, k1, k2, v, lam, lambda_init=0.1, rms_norm=False, dtype=torch.float64)
+    assert torch.equal(x, x2)
+    # scale invariance of the normalised output for mean-square >> eps
+    y3 = orc.forward(q1, q2, k1, k2, 1000.0 * v, lam, lambda_init=li, rms_norm=True, dtype=torch.float64)
+    y4 = orc.forward(q1, q2, k1, k2, 3000.0 * v, lam, lambda_init=li, rms_norm=True, dtype=torch.float64)
+    assert torch.allclose(y3, y4, atol=1e-9)
+    # eps sits inside the square root, added to the mean square
+    tiny = orc.forward(q1, q2, k1, k2, 1e-6 * v, lam, lambda_init=li, rms_norm=True, dtype=torch.float64)
+    assert torch.allclose(tiny, (1 - li) * (1e-6 * x) / math.sqrt(1e-5), rtol=1e-5, atol=0)
+
+
+@pytest.mark.parametrize("rms", [False, True])
+def test_brute_force_f64(rms):
+    q1, q2, k1, k2, v = rand_inputs(1, 1, 7, 3, seed=6)
+    y = orc.forward(q1, q2, k1, k2, v, 0.37, lambda_init=0.6, rms_norm=rms, dtype=torch.float64)
+    ref = brute_force.forward_unit(*(t[0, 0].numpy() for t in (q1, q2, k1, k2, v)), 0.37, 0.6, rms)
+    assert np.allclose(y[0, 0].numpy(), ref, atol=1e-12)
+
+
+def test_aux_outputs():
+    q1, q2, k1, k2, v = rand_inputs(1, 2, 19, 8, seed=7)
+    y, aux = orc.forward(q1, q2, k1, k2, v, 0.3, rms_norm=True, dtype=torch.float64, want_aux=True)
+    s = 1 / math.sqrt(8)
+    assert torch.allclose(aux["lse1"], torch.logsumexp(s * q1 @ k1.transpose(-1, -2), -1), atol=1e-12)
+    assert torch.allclose(aux["lse2"], torch.logsumexp(s * q2 @ k2.transpose(-1, -2), -1), atol=1e-12)
+    assert torch.allclose(aux["u1"], F.scaled_dot_product_attention(q1, k1, v), atol=1e-12)
+    assert torch.allclose(aux["u2"], F.scaled_dot_product_attention(q2, k2, v), atol=1e-12)
+    assert torch.allclose(aux["x"], aux["u1"] - 0.3 * aux["u2"], atol=1e-12)
+    assert torch.allclose(y, 0.2 * aux["x"] * aux["rinv"][..., None], atol=1e-12)
+
+
+@pytest.mark.parametrize("rms", [False, True])
+def test_gradcheck_f64(rms):
+    q1, q2, k1, k2, v = rand_inputs(1, 1, 5, 2, seed=8)
+    lam = torch.tensor(0.45, dtype=torch.float64)
+    ins = [t[0].clone().requires_grad_(True) for t in (q1, q2, k1, k2, v)] + [lam.requires_grad_(True)]
+    fn = lambda a, b, c, d, e, l: orc.forward_unit(a, b, c, d, e, l, 0.8, rms)
+    assert torch.autograd.gradcheck(fn, ins, eps=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("rms", [False, True])
+def test_explicit_backward_matches_autograd(rms):
+    q1, q2, k1, k2, v = rand_inputs(2, 2, 21, 8, seed=9)
+    g = torch.Generator().manual_seed(10)
+    dy = torch.randn(2, 2, 21, 16, generator=g, dtype=torch.float64)
+    lam = torch.tensor([0.55], dtype=torch.float64)
+    auto = orc.forward_backward(q1, q2, k1, k2, v, lam, dy, 0.8, rms, dtype=torch.float64, chunk=3)
+    expl = orc.backward_explicit(q1, q2, k1, k2, v, lam, dy, 0.8, rms, dtype=torch.float64)
+    for a, e in zip(auto[1:], expl):
+        assert torch.allclose(a, e, atol=1e-11), (a - e).abs().max()
+
+
+def test_lambda_zero_grads_match_sdpa():
+    q1, q2, k1, k2, v = rand_inputs(1, 2, 16, 8, seed=11)
+    g = torch.Generator().manual_seed(12)
+    dy = torch.randn(1, 2, 16, 16, generator=g, dtype=torch.float64)
+    out = orc.forward_backward(q1, q2, k1, k2, v, 0.0, dy, rms_norm=False, dtype=torch.float64)
+    a, b, c = (t.clone().requires_grad_(True) for t in (q1, k1, v))
+    ref = torch.autograd.grad(F.scaled_dot_product_attention(a, b, c), (a, b, c), dy)
+    assert torch.allclose(out[1], ref[0], atol=1e-12)
+    assert torch.allclose(out[3], ref[1], atol=1e-12)
+    assert torch.allclose(out[5], ref[2], atol=1e-12)
+    assert torch.count_nonzero(out[2]) == 0 and torch.count_nonzero(out[4]) == 0
+    # d(lambda) = -sum(dX * U2) is still non-zero at lambda = 0
+    u2 = F.scaled_dot_product_attention(q2, k2, v)
+    assert torch.allclose(out[6], -(dy * u2).sum().reshape(1), atol=1e-11)
+
+
+@pytest.mark.parametrize("rms", [False, True])
+def test_dlambda_finite_difference(rms):
+    q1, q2, k1, k2, v = rand_inputs(1, 2, 12, 4, seed=13)
+    g = torch.Generator().manual_seed(14)
+    dy = torch.randn(1, 2, 12, 8, generator=g, dtype=torch.float64)
+    lam, h = 0.5, 1e-6
+    out = orc.forward_backward(q1, q2, k1, k2, v, lam, dy, 0.8, rms, dtype=torch.float64)
+    yp = orc.forward(q1, q2, k1, k2, v, lam + h, 0.8, rms, dtype=torch.float64)
+    ym = orc.forward(q1, q2, k1, k2, v, lam - h, 0.8, rms, dtype=torch.float64)
+    fd = ((yp - ym) * dy).sum() / (2 * h)
+    assert abs(out[6].item() - fd.item()) < 1e-6 * max(1.0, abs(fd.item()))
+
+
+def test_chunking_and_dtype():
+    q1, q2, k1, k2, v = rand_inputs(2, 3, 16, 8, seed=15, dtype=torch.float16)
+    a = orc.forward(q1, q2, k1, k2, v, 0.5, rms_norm=True, chunk=1)
+    b = orc.forward(q1, q2, k1, k2, v, 0.5, rms_norm=True, chunk=6)
+    assert a.dtype == torch.float32 and torch.allclose(a, b, atol=1e-6)
+    lam = torch.tensor([0.5], dtype=torch.float16)
+    c = orc.forward(q1, q2, k1, k2, v, lam, rms_norm=True)
+    assert torch.allclose(a, c, atol=1e-6)
