@@ -1,0 +1,83 @@
+/*
+ * libdiffattn -- C ABI of the MI355X (gfx950) differential-attention kernels.
+ *
+ * This is the device-call boundary of the path `layers.MultiheadDiffAttnKernel` ->
+ * `kernel._diff_attention.forward/backward` -> kernel launch.  In the reference that boundary is
+ * the pair of Triton launches `diff_attn_fwd[grid](...)` (src/kernel.py:476-503) and
+ * `diff_attn_bwd[grid](...)` (src/kernel.py:531-570); the entry points below take the same
+ * operands as plain device pointers and sizes.
+ *
+ * Conventions (all entry points):
+ *   - every tensor is dense row-major fp16 ("half"), [B,H,N,D] for q1,q2,k1,k2 and their
+ *     gradients, [B,H,N,2D] for v, y, u2, dy, dv; row statistics are fp32 [B,H,N];
+ *   - D is 32, 64 or 128; N is a multiple of 128;
+ *   - lambda_scale is a DEVICE pointer to one fp16 value (the reference loads it in-kernel,
+ *     src/kernel.py:138);
+ *   - `stream` is a hipStream_t passed as void*; work is only enqueued on it.  No entry point
+ *     allocates, frees, synchronises or keeps global state; all are re-entrant;
+ *   - return value: 0 on success, a negative DIFFATTN_E* code for rejected arguments, or a
+ *     positive hipError_t value if a launch failed.
+ */
+#ifndef DIFFATTN_H_
+#define DIFFATTN_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DIFFATTN_OK 0
+#define DIFFATTN_EINVAL_NULL (-1)   /* a required pointer is null */
+#define DIFFATTN_EINVAL_DIM (-2)    /* D not in {32,64,128} or B,H,N not positive */
+#define DIFFATTN_EINVAL_SEQ (-3)    /* N not a multiple of 128 */
+#define DIFFATTN_EINVAL_WS (-4)     /* workspace too small */
+#define DIFFATTN_EINVAL_ALIGN (-5)  /* a pointer is not 16-byte aligned */
+
+/* ABI version of this header; bumped when a signature changes. */
+int diffattn_abi_version(void);
+
+/* Human-readable text for a return code of this library (static storage). */
+const char* diffattn_strerror(int code);
+
+/*
+ * Forward.  Replaces the launch of diff_attn_fwd (src/kernel.py:476-503).
+ *   y    [B,H,N,2D]  out: (softmax(s q1 k1^T) - lambda softmax(s q2 k2^T)) v, then, iff rms_norm,
+ *                    (1 - lambda_init) * rmsnorm(.) with eps 1e-5 (src/kernel.py:188-198)
+ *   u2   [B,H,N,2D]  out, optional (may be NULL when no backward follows): softmax(s q2 k2^T) v
+ *   lse1, lse2 [B,H,N] fp32 out, optional: natural-log row logsumexp of the scaled scores
+ *                    (the reference's M1/M2, src/kernel.py:188-189,203-204)
+ *   rinv [B,H,N] fp32 out, optional, written only when rms_norm: rsqrt(mean(x^2) + 1e-5)
+ * The reference additionally stores both per-stream outputs O1,O2 (src/kernel.py:205-206); here
+ * the backward rebuilds the pre-norm row from y and rinv, so only u2 is kept.
+ */
+int diffattn_forward(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                     const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
+                     int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                     void* stream);
+
+/* Bytes of device workspace diffattn_backward needs for this problem size (0 on bad sizes). */
+size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D);
+
+/*
+ * Backward.  Replaces the launch of diff_attn_bwd (src/kernel.py:531-570) and the host-side
+ * reduction of the lambda gradient (src/kernel.py:573).
+ *   inputs : q1,q2,k1,k2,v,lambda_scale as in forward; y,u2,lse1,lse2,rinv as written by forward
+ *            (rinv is ignored unless rms_norm); dy [B,H,N,2D] upstream gradient, dense.
+ *   outputs: dq1,dq2,dk1,dk2 [B,H,N,D], dv [B,H,N,2D] fp16; dlambda: one fp16 value, DEVICE
+ *            memory, written (not accumulated), reduced in a fixed order: bit-reproducible.
+ *   workspace: device memory of at least diffattn_backward_workspace_bytes(B,H,N,D) bytes,
+ *            256-byte aligned, contents undefined before and after.
+ */
+int diffattn_backward(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                      const void* lambda_scale, const void* y, const void* u2,
+                      const float* lse1, const float* lse2, const float* rinv, const void* dy,
+                      void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
+                      void* workspace, size_t workspace_bytes,
+                      int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                      void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DIFFATTN_H_ */

@@ -1,0 +1,67 @@
+"""GPU parity: the HIP kernels, called through layers.MultiheadDiffAttnKernel -> C ABI, against
+the fp32 CPU oracle on the same seeded inputs."""
+import pytest
+import torch
+
+from oracle import diff_attn_oracle as orc
+from util import GRAD_RTOL, Y_ATOL, make_inputs, max_abs, rel_to_max, run_kernel
+
+pytestmark = pytest.mark.gpu
+
+GRAD_NAMES = ("dq1", "dq2", "dk1", "dk2", "dv", "dlambda")
+
+
+def check_case(B, H, N, D, seed, lam, lambda_init, rms, scale=1.0, backward=True):
+    q1, q2, k1, k2, v, dy = make_inputs(B, H, N, D, seed, scale)
+    print("case", dict(B=B, H=H, N=N, D=D, seed=seed, lam=lam, rms=rms, backward=backward), flush=True)
+    y, grads = run_kernel(q1, q2, k1, k2, v, lam, lambda_init, rms, dy if backward else None)
+    lam16 = torch.tensor([lam], dtype=torch.float16)
+    if backward:
+        ref = orc.forward_backward(q1, q2, k1, k2, v, lam16, dy, lambda_init, rms)
+    else:
+        ref = (orc.forward(q1, q2, k1, k2, v, lam16, lambda_init, rms),)
+    err_y = max_abs(y, ref[0])
+    print("  y max-abs err %.3e" % err_y, flush=True)
+    assert torch.isfinite(y).all()
+    assert err_y <= Y_ATOL
+    if backward:
+        for name, gk, gr in zip(GRAD_NAMES, grads, ref[1:]):
+            e = rel_to_max(gk, gr)
+            print("  %s rel-to-max err %.3e (ref max %.3e)" % (name, e, gr.abs().max().item()), flush=True)
+            assert torch.isfinite(gk).all(), name
+            assert e <= GRAD_RTOL, name
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("rms", [True, False])
+def test_small_forward_backward(D, rms):
+    check_case(1, 2, 256, D, seed=100 + D, lam=0.5, lambda_init=0.8, rms=rms)
+
+
+@pytest.mark.parametrize("D,N", [(32, 128), (64, 384), (128, 128), (64, 640)])
+def test_odd_tile_counts(D, N):
+    check_case(2, 1, N, D, seed=7 * D + N, lam=0.3, lambda_init=0.5, rms=True)
+
+
+def test_config0_forward():
+    # BASELINE config 0: B=2 H=16 N=512 D=32, lambda 0.5, lambda_init 0.8, rms_norm on, forward only
+    check_case(2, 16, 512, 32, seed=0, lam=0.5, lambda_init=0.8, rms=True, backward=False)
+
+
+def test_config1_forward_backward():
+    # BASELINE config 1: same shape and inputs as config 0, forward + backward
+    check_case(2, 16, 512, 32, seed=0, lam=0.5, lambda_init=0.8, rms=True, backward=True)
+
+
+def test_negative_and_zero_lambda():
+    check_case(1, 2, 256, 64, seed=5, lam=-0.5, lambda_init=0.8, rms=True)
+    check_case(1, 2, 256, 64, seed=6, lam=0.0, lambda_init=0.8, rms=False)
+
+
+def test_backward_is_deterministic():
+    q1, q2, k1, k2, v, dy = make_inputs(2, 4, 512, 64, seed=11)
+    a = run_kernel(q1, q2, k1, k2, v, 0.5, 0.8, True, dy)
+    b = run_kernel(q1, q2, k1, k2, v, 0.5, 0.8, True, dy)
+    assert torch.equal(a[0], b[0])
+    for ga, gb in zip(a[1], b[1]):
+        assert torch.equal(ga, gb)

@@ -1,0 +1,42 @@
+"""Shared helpers of the parity tests: seeded synthetic inputs and the tolerance metrics."""
+import torch
+
+# tolerances stated by the build's target: outputs within max-abs 2e-2 of the fp32 oracle,
+# gradients within 5e-2 relative to the max-norm of the oracle gradient
+Y_ATOL = 2e-2
+GRAD_RTOL = 5e-2
+
+
+def make_inputs(B, H, N, D, seed, scale=1.0, with_dy=True):
+    """fp16 tensors drawn i.i.d. N(0, scale^2) on the CPU in the fixed order q1,q2,k1,k2,v,dy."""
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda d: (torch.randn(B, H, N, d, generator=g, dtype=torch.float32) * scale).to(torch.float16)
+    q1, q2, k1, k2 = mk(D), mk(D), mk(D), mk(D)
+    v = mk(2 * D)
+    dy = (torch.randn(B, H, N, 2 * D, generator=g, dtype=torch.float32)).to(torch.float16) if with_dy else None
+    return q1, q2, k1, k2, v, dy
+
+
+def max_abs(a, b):
+    return (a.float().cpu() - b.float().cpu()).abs().max().item()
+
+
+def rel_to_max(a, ref):
+    ref = ref.float().cpu()
+    return (a.float().cpu() - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
+
+
+def run_kernel(q1, q2, k1, k2, v, lam_value, lambda_init, rms_norm, dy=None, device="cuda"):
+    """Runs layers.MultiheadDiffAttnKernel on the GPU; returns (y, grads or None) as CPU tensors."""
+    from layers import MultiheadDiffAttnKernel
+
+    need = dy is not None
+    t = [x.to(device).requires_grad_(need) for x in (q1, q2, k1, k2, v)]
+    lam = torch.tensor([lam_value], dtype=torch.float16, device=device, requires_grad=need)
+    y = MultiheadDiffAttnKernel(*t, lambda_scale=lam, lambda_init=lambda_init, rms_norm=rms_norm)
+    grads = None
+    if need:
+        y.backward(dy.to(device))
+        grads = [x.grad.cpu() for x in t] + [lam.grad.cpu()]
+    torch.cuda.synchronize()
+    return y.detach().cpu(), grads

@@ -1,0 +1,53 @@
+"""ctypes binding of libdiffattn.so (C ABI in include/diffattn.h).
+
+torch is imported first on purpose: the library resolves the HIP runtime by soname, so it shares
+the runtime (and therefore streams and device pointers) that torch has already loaded.
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (must precede loading the library)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libdiffattn.so")
+
+_lib = None
+
+_vp = ctypes.c_void_p
+_fp = ctypes.c_void_p  # float* passed as raw addresses
+
+SYMBOLS = {
+    "diffattn_abi_version": (ctypes.c_int, []),
+    "diffattn_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "diffattn_forward": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp] + [ctypes.c_int] * 4
+                         + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
+    "diffattn_backward_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 4),
+    "diffattn_backward": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp, _vp] + [_vp] * 6
+                          + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 4
+                          + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
+}
+
+
+class NativeLibraryMissing(RuntimeError):
+    pass
+
+
+def lib():
+    """Returns the loaded library; raises if it has not been built (there is no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise NativeLibraryMissing(
+                "libdiffattn.so is not built: run `python %s`" % os.path.join(_HERE, "build.py"))
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(code):
+    if code != 0:
+        raise RuntimeError("libdiffattn: %s (code %d)" % (lib().diffattn_strerror(code).decode(), code))

@@ -1,0 +1,110 @@
+// C-ABI entry points of libdiffattn (declared in include/diffattn.h): argument validation,
+// workspace carve-up and kernel launches.  Nothing here allocates, synchronises or keeps state.
+#include "../../include/diffattn.h"
+#include "params.hpp"
+
+using namespace da;
+
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_dims(int B, int H, int N, int D) {
+  if (B <= 0 || H <= 0 || N <= 0) return DIFFATTN_EINVAL_DIM;
+  if (D != 32 && D != 64 && D != 128) return DIFFATTN_EINVAL_DIM;
+  if ((long long)B * H > 0x7fffffffLL / 64) return DIFFATTN_EINVAL_DIM;
+  if (N % 128 != 0) return DIFFATTN_EINVAL_SEQ;
+  return DIFFATTN_OK;
+}
+
+inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+struct WsLayout {
+  size_t dx, stat, part, total;
+};
+
+WsLayout ws_layout(int BH, int N, int D) {
+  WsLayout w;
+  size_t rows = (size_t)BH * N;
+  size_t off = 0;
+  w.dx = off;      off = round_up(off + rows * 2 * D * sizeof(half_t), 256);
+  w.stat = off;    off = round_up(off + 4 * rows * sizeof(float), 256);
+  w.part = off;    off = round_up(off + (size_t)bwd_num_partials(BH, N, D) * sizeof(float), 256);
+  w.total = off;
+  return w;
+}
+
+}  // namespace
+
+extern "C" {
+
+int diffattn_abi_version(void) { return 1; }
+
+const char* diffattn_strerror(int code) {
+  switch (code) {
+    case DIFFATTN_OK: return "success";
+    case DIFFATTN_EINVAL_NULL: return "a required pointer is null";
+    case DIFFATTN_EINVAL_DIM: return "unsupported sizes: D must be 32, 64 or 128 and B, H, N positive";
+    case DIFFATTN_EINVAL_SEQ: return "N must be a multiple of 128";
+    case DIFFATTN_EINVAL_WS: return "workspace too small or misaligned";
+    case DIFFATTN_EINVAL_ALIGN: return "tensor pointers must be 16-byte aligned";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+  return "unknown diffattn error";
+}
+
+int diffattn_forward(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                     const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
+                     int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                     void* stream) {
+  if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y) return DIFFATTN_EINVAL_NULL;
+  if (int e = check_dims(B, H, N, D)) return e;
+  if (!aligned16(q1) || !aligned16(q2) || !aligned16(k1) || !aligned16(k2) || !aligned16(v) ||
+      !aligned16(y) || !aligned16(u2))
+    return DIFFATTN_EINVAL_ALIGN;
+  FwdParams p;
+  p.q1 = (const half_t*)q1; p.q2 = (const half_t*)q2; p.k1 = (const half_t*)k1; p.k2 = (const half_t*)k2;
+  p.v = (const half_t*)v; p.lambda_scale = (const half_t*)lambda_scale;
+  p.y = (half_t*)y; p.u2 = (half_t*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
+  p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = rms_norm ? 1 : 0;
+  return (int)launch_fwd(p, D, (hipStream_t)stream);
+}
+
+size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D) {
+  if (check_dims(B, H, N, D)) return 0;
+  return ws_layout(B * H, N, D).total;
+}
+
+int diffattn_backward(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                      const void* lambda_scale, const void* y, const void* u2,
+                      const float* lse1, const float* lse2, const float* rinv, const void* dy,
+                      void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
+                      void* workspace, size_t workspace_bytes,
+                      int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                      void* stream) {
+  if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy ||
+      !dq1 || !dq2 || !dk1 || !dk2 || !dv || !dlambda || !workspace)
+    return DIFFATTN_EINVAL_NULL;
+  if (rms_norm && !rinv) return DIFFATTN_EINVAL_NULL;
+  if (int e = check_dims(B, H, N, D)) return e;
+  const void* ptrs[] = {q1, q2, k1, k2, v, y, u2, dy, dq1, dq2, dk1, dk2, dv};
+  for (const void* q : ptrs)
+    if (!aligned16(q)) return DIFFATTN_EINVAL_ALIGN;
+  const WsLayout w = ws_layout(B * H, N, D);
+  if (workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return DIFFATTN_EINVAL_WS;
+  char* ws = (char*)workspace;
+  BwdParams p;
+  p.q1 = (const half_t*)q1; p.q2 = (const half_t*)q2; p.k1 = (const half_t*)k1; p.k2 = (const half_t*)k2;
+  p.v = (const half_t*)v; p.lambda_scale = (const half_t*)lambda_scale;
+  p.y = (const half_t*)y; p.u2 = (const half_t*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
+  p.dy = (const half_t*)dy;
+  p.dq1 = (half_t*)dq1; p.dq2 = (half_t*)dq2; p.dk1 = (half_t*)dk1; p.dk2 = (half_t*)dk2; p.dv = (half_t*)dv;
+  p.dlambda = (half_t*)dlambda;
+  p.dx = (half_t*)(ws + w.dx); p.stat = (float*)(ws + w.stat);
+  p.dlam_part = (float*)(ws + w.part); p.n_part = bwd_num_partials(B * H, N, D);
+  p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = rms_norm ? 1 : 0;
+  return (int)launch_bwd(p, D, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,477 @@
+// Differential-attention backward for gfx950.  Same mathematics as the reference's fused backward
+// (src/kernel.py:221-458) but split into stream-ordered kernels, which removes the reference's
+// in-launch dependency between the row preprocess and the main loops:
+//
+//   bwd_prep_kernel   per row: RMSNorm backward (src/kernel.py:283-290), the two row dots
+//                     delta1/delta2 (:295-296), d(lambda) partials (:293); writes dX in fp16 and
+//                     the four row statistics the main kernels need.
+//   bwd_dkdv_kernel   one workgroup per 128 keys, loops over all query tiles:
+//                     dV += (P1 - lambda P2)^T dX, dK_t += s dS_t^T Q_t      (:410-424)
+//   bwd_dq_kernel     one workgroup per 128 queries, loops over all key tiles:
+//                     dQ_t += s dS_t K_t                                      (:426-436)
+//   bwd_dlambda_kernel  fixed-order sum of the partials into one fp16 value   (:573)
+//
+// The pre-norm row X is rebuilt as Y / ((1 - lambda_init) * rinv); only U2 = softmax(S2) V is
+// needed besides it, because U1 = X + lambda U2.
+#include "params.hpp"
+
+namespace da {
+
+constexpr int kPrepRows = 64;   // rows per workgroup of the preprocess kernel = one d(lambda) partial
+
+int bwd_num_partials(int BH, int N, int D) { (void)D; return (int)(((long long)BH * N) / kPrepRows); }
+
+// ------------------------------------------------------------------------------------------------
+template <int D, bool RMS>
+__global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
+  constexpr int DV = 2 * D, LPR = DV / 8, RPP = 256 / LPR;
+  __shared__ float red[256];
+  const int tid = threadIdx.x, sub = tid % LPR, rloc = tid / LPR;
+  const float lam = (float)p.lambda_scale[0];
+  const float c = 1.0f - p.lambda_init;
+  const size_t rows = (size_t)p.BH * p.N;
+  float part = 0.f;
+#pragma unroll 1
+  for (int pass = 0; pass < kPrepRows / RPP; ++pass) {
+    const size_t row = (size_t)blockIdx.x * kPrepRows + pass * RPP + rloc;
+    const size_t off = row * DV + 8 * sub;
+    const h8 y8 = *reinterpret_cast<const h8*>(p.y + off);
+    const h8 u8 = *reinterpret_cast<const h8*>(p.u2 + off);
+    const h8 g8 = *reinterpret_cast<const h8*>(p.dy + off);
+    float dx[8], x[8];
+    if (RMS) {
+      float gy = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) gy += (float)g8[e] * (float)y8[e];
+#pragma unroll
+      for (int msk = LPR / 2; msk >= 1; msk >>= 1) gy += __shfl_xor(gy, msk, 64);
+      const float r = p.rinv[row];
+      if (c != 0.f) {
+        const float a = c * r, b = r * gy / (c * DV), ix = 1.0f / (c * r);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          dx[e] = a * (float)g8[e] - b * (float)y8[e];
+          x[e] = (float)y8[e] * ix;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { dx[e] = 0.f; x[e] = 0.f; }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { dx[e] = (float)g8[e]; x[e] = (float)y8[e]; }
+    }
+    float t2 = 0.f, tx = 0.f;
+    h8 d8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      t2 += dx[e] * (float)u8[e];
+      tx += dx[e] * x[e];
+      d8[e] = (half_t)dx[e];
+    }
+#pragma unroll
+    for (int msk = LPR / 2; msk >= 1; msk >>= 1) {
+      t2 += __shfl_xor(t2, msk, 64);
+      tx += __shfl_xor(tx, msk, 64);
+    }
+    *reinterpret_cast<h8*>(p.dx + off) = d8;
+    if (sub == 0) {
+      const float delta2 = -lam * t2;
+      p.stat[0 * rows + row] = -p.lse1[row] * kLog2e;
+      p.stat[1 * rows + row] = -p.lse2[row] * kLog2e;
+      p.stat[2 * rows + row] = tx - delta2;
+      p.stat[3 * rows + row] = delta2;
+      part -= t2;
+    }
+  }
+  red[tid] = part;
+  __syncthreads();
+#pragma unroll
+  for (int s = 128; s >= 1; s >>= 1) {
+    if (tid < s) red[tid] += red[tid + s];
+    __syncthreads();
+  }
+  if (tid == 0) p.dlam_part[blockIdx.x] = red[0];
+}
+
+__global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restrict__ part, int n, half_t* out) {
+  __shared__ float red[256];
+  const int tid = threadIdx.x;
+  float acc = 0.f;
+  for (int i = tid; i < n; i += 256) acc += part[i];
+  red[tid] = acc;
+  __syncthreads();
+#pragma unroll
+  for (int s = 128; s >= 1; s >>= 1) {
+    if (tid < s) red[tid] += red[tid + s];
+    __syncthreads();
+  }
+  if (tid == 0) out[0] = (half_t)red[0];
+}
+
+// ------------------------------------------------------------------------------------------------
+template <int D>
+struct DkvCfg {
+  static constexpr int DV = 2 * D;
+  static constexpr int NT = 256;
+  static constexpr int BK = 128;               // keys per workgroup (32 per wave)
+  static constexpr int BQ = 64;                // query rows per staged tile
+  static constexpr int QS = D + 8;             // LDS row strides (halfs)
+  static constexpr int XS = DV + 8;
+  static constexpr int Q_TILE = BQ * QS;
+  static constexpr int X_TILE = BQ * XS;
+  static constexpr int STAT = 4 * BQ * 2;      // 4 float arrays, counted in halfs
+  static constexpr int STAGE = 2 * Q_TILE + X_TILE + STAT;
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void bwd_dkdv_kernel(BwdParams p) {
+  using C = DkvCfg<D>;
+  constexpr int DV = C::DV, NT = C::NT, BK = C::BK, BQ = C::BQ, QS = C::QS, XS = C::XS;
+  constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32, NVT = DV / 32;
+
+  __shared__ __attribute__((aligned(16))) half_t smem[2 * C::STAGE];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int j = lane & 31, g = lane >> 5;
+
+  const int n_kt = p.N / BK;
+  const int tile = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = tile / n_kt, kt = tile % n_kt;
+  const size_t rows = (size_t)p.BH * p.N;
+  const size_t row0 = (size_t)bh * p.N;
+  const int key = kt * BK + wave * 32 + j;
+
+  const float c = p.sm_scale * kLog2e;
+  const float lam = (float)p.lambda_scale[0];
+
+  // persistent B operands: this lane's key row of K1, K2, V
+  h8 kf1[NKS], kf2[NKS], vf[NKV];
+  {
+    const half_t* r1 = p.k1 + (row0 + key) * D + 8 * g;
+    const half_t* r2 = p.k2 + (row0 + key) * D + 8 * g;
+    const half_t* rv = p.v + (row0 + key) * DV + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      kf1[ks] = *reinterpret_cast<const h8*>(r1 + 16 * ks);
+      kf2[ks] = *reinterpret_cast<const h8*>(r2 + 16 * ks);
+    }
+#pragma unroll
+    for (int kv = 0; kv < NKV; ++kv) vf[kv] = *reinterpret_cast<const h8*>(rv + 16 * kv);
+  }
+
+  f16v dv[NVT], dk1[NDT], dk2[NDT];
+#pragma unroll
+  for (int t = 0; t < NVT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dv[t][r] = 0.f;
+#pragma unroll
+  for (int t = 0; t < NDT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dk1[t][r] = 0.f; dk2[t][r] = 0.f; }
+
+  TileStage<BQ, D, QS, NT> stQ1, stQ2;
+  TileStage<BQ, DV, XS, NT> stX;
+  float st_stat = 0.f;
+  const half_t* gq1 = p.q1 + row0 * D;
+  const half_t* gq2 = p.q2 + row0 * D;
+  const half_t* gx = p.dx + row0 * DV;
+  // thread t stages stat[t / BQ][t % BQ]  (4 * BQ = 256 = NT values)
+  const float* gstat = p.stat + (size_t)(tid / BQ) * rows + row0 + (tid % BQ);
+
+  auto stage_load = [&](int qt) {
+    stQ1.load(gq1 + (size_t)qt * BQ * D, tid);
+    stQ2.load(gq2 + (size_t)qt * BQ * D, tid);
+    stX.load(gx + (size_t)qt * BQ * DV, tid);
+    st_stat = gstat[(size_t)qt * BQ];
+  };
+  auto stage_store = [&](int buf) {
+    half_t* b = smem + buf * C::STAGE;
+    stQ1.store(b, tid);
+    stQ2.store(b + C::Q_TILE, tid);
+    stX.store(b + 2 * C::Q_TILE, tid);
+    reinterpret_cast<float*>(b + 2 * C::Q_TILE + C::X_TILE)[tid] = st_stat;
+  };
+
+  stage_load(0);
+  stage_store(0);
+  __syncthreads();
+
+  // per-lane LDS offsets (halfs)
+  const int a_q = j * QS + 8 * g;                 // A fragment of Q (row = query j)
+  const int a_x = j * XS + 8 * g;                 // A fragment of dX
+  const int tr_row = 4 * g + ((lane & 15) >> 2);  // transposing reads: row inside a 16-row k-step
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  const int n_qt = p.N / BQ;
+  for (int qt = 0; qt < n_qt; ++qt) {
+    const half_t* sQ1 = smem + (qt & 1) * C::STAGE;
+    const half_t* sQ2 = sQ1 + C::Q_TILE;
+    const half_t* sX = sQ1 + 2 * C::Q_TILE;
+    const float* sStat = reinterpret_cast<const float*>(sQ1 + 2 * C::Q_TILE + C::X_TILE);
+    const bool more = (qt + 1 < n_qt);
+    if (more) stage_load(qt + 1);
+
+#pragma unroll
+    for (int qs = 0; qs < BQ / 32; ++qs) {
+      f16v s1, s2, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { s1[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        h8 a1 = *reinterpret_cast<const h8*>(sQ1 + qs * 32 * QS + a_q + 16 * ks);
+        s1 = mfma32(a1, kf1[ks], s1);
+        h8 a2 = *reinterpret_cast<const h8*>(sQ2 + qs * 32 * QS + a_q + 16 * ks);
+        s2 = mfma32(a2, kf2[ks], s2);
+      }
+#pragma unroll
+      for (int kv = 0; kv < NKV; ++kv) {
+        h8 a = *reinterpret_cast<const h8*>(sX + qs * 32 * XS + a_x + 16 * kv);
+        dp = mfma32(a, vf[kv], dp);
+      }
+      // registers r of the 32x32 tiles hold query rows 8*(r/4) + 4g + (r%4)
+      h8 pc[2], d1[2], d2[2];
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int qo = qs * 32 + 8 * r4 + 4 * g;
+        const f4v nl1 = *reinterpret_cast<const f4v*>(sStat + 0 * BQ + qo);
+        const f4v nl2 = *reinterpret_cast<const f4v*>(sStat + 1 * BQ + qo);
+        const f4v de1 = *reinterpret_cast<const f4v*>(sStat + 2 * BQ + qo);
+        const f4v de2 = *reinterpret_cast<const f4v*>(sStat + 3 * BQ + qo);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * r4 + e;
+          const float p1 = fast_exp2(__builtin_fmaf(s1[r], c, nl1[e]));
+          const float p2 = fast_exp2(__builtin_fmaf(s2[r], c, nl2[e]));
+          const float ds1 = p1 * (dp[r] - de1[e]);
+          const float ds2 = p2 * (-lam * dp[r] - de2[e]);
+          pc[r / 8][r % 8] = (half_t)(p1 - lam * p2);
+          d1[r / 8][r % 8] = (half_t)ds1;
+          d2[r / 8][r % 8] = (half_t)ds2;
+        }
+      }
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const int rbase = qs * 32 + 16 * kk + tr_row;
+#pragma unroll
+        for (int tt = 0; tt < NVT; ++tt) {
+          const half_t* bp = sX + rbase * XS + 32 * tt + tr_col;
+          h8 b = join(lds_read_tr(bp), lds_read_tr(bp + 8 * XS));
+          dv[tt] = mfma32(pc[kk], b, dv[tt]);
+        }
+#pragma unroll
+        for (int tt = 0; tt < NDT; ++tt) {
+          const half_t* b1p = sQ1 + rbase * QS + 32 * tt + tr_col;
+          h8 b1 = join(lds_read_tr(b1p), lds_read_tr(b1p + 8 * QS));
+          dk1[tt] = mfma32(d1[kk], b1, dk1[tt]);
+          const half_t* b2p = sQ2 + rbase * QS + 32 * tt + tr_col;
+          h8 b2 = join(lds_read_tr(b2p), lds_read_tr(b2p + 8 * QS));
+          dk2[tt] = mfma32(d2[kk], b2, dk2[tt]);
+        }
+      }
+    }
+
+    if (more) stage_store((qt + 1) & 1);
+    __syncthreads();
+  }
+
+  // accumulator tile tt: column = 32*tt + j (feature), register r = key row 8*(r/4) + 4g + (r%4)
+  const size_t krow0 = row0 + (size_t)kt * BK + wave * 32;
+#pragma unroll
+  for (int tt = 0; tt < NVT; ++tt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kr = 8 * (r / 4) + 4 * g + (r % 4);
+      p.dv[(krow0 + kr) * DV + 32 * tt + j] = (half_t)dv[tt][r];
+    }
+#pragma unroll
+  for (int tt = 0; tt < NDT; ++tt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kr = 8 * (r / 4) + 4 * g + (r % 4);
+      p.dk1[(krow0 + kr) * D + 32 * tt + j] = (half_t)(dk1[tt][r] * p.sm_scale);
+      p.dk2[(krow0 + kr) * D + 32 * tt + j] = (half_t)(dk2[tt][r] * p.sm_scale);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+template <int D>
+struct DqCfg {
+  static constexpr int DV = 2 * D;
+  static constexpr int NT = 256;
+  static constexpr int BM = 128;               // query rows per workgroup (32 per wave)
+  static constexpr int BN = (D <= 64) ? 64 : 32;  // keys per staged tile
+  static constexpr int KS = D + 8;
+  static constexpr int VS = DV + 8;
+  static constexpr int K_TILE = BN * KS;
+  static constexpr int V_TILE = BN * VS;
+  static constexpr int STAGE = 2 * K_TILE + V_TILE;
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void bwd_dq_kernel(BwdParams p) {
+  using C = DqCfg<D>;
+  constexpr int DV = C::DV, NT = C::NT, BM = C::BM, BN = C::BN, KS = C::KS, VS = C::VS;
+  constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
+
+  __shared__ __attribute__((aligned(16))) half_t smem[2 * C::STAGE];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int j = lane & 31, g = lane >> 5;
+
+  const int n_qt = p.N / BM;
+  const int tile = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = tile / n_qt, qt = tile % n_qt;
+  const size_t rows = (size_t)p.BH * p.N;
+  const size_t row0 = (size_t)bh * p.N;
+  const size_t qrow = row0 + qt * BM + wave * 32 + j;
+
+  const float c = p.sm_scale * kLog2e;
+  const float lam = (float)p.lambda_scale[0];
+
+  // persistent B operands: this lane's query row of Q1, Q2, dX, and its row statistics
+  h8 qf1[NKS], qf2[NKS], xf[NKV];
+  {
+    const half_t* r1 = p.q1 + qrow * D + 8 * g;
+    const half_t* r2 = p.q2 + qrow * D + 8 * g;
+    const half_t* rx = p.dx + qrow * DV + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      qf1[ks] = *reinterpret_cast<const h8*>(r1 + 16 * ks);
+      qf2[ks] = *reinterpret_cast<const h8*>(r2 + 16 * ks);
+    }
+#pragma unroll
+    for (int kv = 0; kv < NKV; ++kv) xf[kv] = *reinterpret_cast<const h8*>(rx + 16 * kv);
+  }
+  const float nl1 = p.stat[0 * rows + qrow], nl2 = p.stat[1 * rows + qrow];
+  const float de1 = p.stat[2 * rows + qrow], de2 = p.stat[3 * rows + qrow];
+
+  f16v dq1[NDT], dq2[NDT];
+#pragma unroll
+  for (int t = 0; t < NDT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dq1[t][r] = 0.f; dq2[t][r] = 0.f; }
+
+  TileStage<BN, D, KS, NT> stK1, stK2;
+  TileStage<BN, DV, VS, NT> stV;
+  const half_t* gk1 = p.k1 + row0 * D;
+  const half_t* gk2 = p.k2 + row0 * D;
+  const half_t* gv = p.v + row0 * DV;
+
+  stK1.load(gk1, tid); stK2.load(gk2, tid); stV.load(gv, tid);
+  stK1.store(smem, tid); stK2.store(smem + C::K_TILE, tid); stV.store(smem + 2 * C::K_TILE, tid);
+  __syncthreads();
+
+  const int a_k = j * KS + 8 * g;                 // A fragment of K (row = key j)
+  const int a_v = j * VS + 8 * g;                 // A fragment of V
+  const int tr_row = 4 * g + ((lane & 15) >> 2);
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  const int n_tiles = p.N / BN;
+  for (int t = 0; t < n_tiles; ++t) {
+    const half_t* sK1 = smem + (t & 1) * C::STAGE;
+    const half_t* sK2 = sK1 + C::K_TILE;
+    const half_t* sV = sK1 + 2 * C::K_TILE;
+    const bool more = (t + 1 < n_tiles);
+    if (more) {
+      stK1.load(gk1 + (size_t)(t + 1) * BN * D, tid);
+      stK2.load(gk2 + (size_t)(t + 1) * BN * D, tid);
+      stV.load(gv + (size_t)(t + 1) * BN * DV, tid);
+    }
+
+#pragma unroll
+    for (int ksub = 0; ksub < BN / 32; ++ksub) {
+      // transposed tiles [32 keys x 32 queries]: this lane's column is its query
+      f16v s1, s2, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { s1[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        h8 a1 = *reinterpret_cast<const h8*>(sK1 + ksub * 32 * KS + a_k + 16 * ks);
+        s1 = mfma32(a1, qf1[ks], s1);
+        h8 a2 = *reinterpret_cast<const h8*>(sK2 + ksub * 32 * KS + a_k + 16 * ks);
+        s2 = mfma32(a2, qf2[ks], s2);
+      }
+#pragma unroll
+      for (int kv = 0; kv < NKV; ++kv) {
+        h8 a = *reinterpret_cast<const h8*>(sV + ksub * 32 * VS + a_v + 16 * kv);
+        dp = mfma32(a, xf[kv], dp);
+      }
+      h8 b1[2], b2[2];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p1 = fast_exp2(__builtin_fmaf(s1[r], c, nl1));
+        const float p2 = fast_exp2(__builtin_fmaf(s2[r], c, nl2));
+        b1[r / 8][r % 8] = (half_t)(p1 * (dp[r] - de1));
+        b2[r / 8][r % 8] = (half_t)(p2 * (-lam * dp[r] - de2));
+      }
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const int rbase = ksub * 32 + 16 * kk + tr_row;
+#pragma unroll
+        for (int tt = 0; tt < NDT; ++tt) {
+          const half_t* a1p = sK1 + rbase * KS + 32 * tt + tr_col;
+          h8 a1 = join(lds_read_tr(a1p), lds_read_tr(a1p + 8 * KS));
+          dq1[tt] = mfma32(a1, b1[kk], dq1[tt]);
+          const half_t* a2p = sK2 + rbase * KS + 32 * tt + tr_col;
+          h8 a2 = join(lds_read_tr(a2p), lds_read_tr(a2p + 8 * KS));
+          dq2[tt] = mfma32(a2, b2[kk], dq2[tt]);
+        }
+      }
+    }
+
+    if (more) {
+      half_t* nb = smem + ((t + 1) & 1) * C::STAGE;
+      stK1.store(nb, tid); stK2.store(nb + C::K_TILE, tid); stV.store(nb + 2 * C::K_TILE, tid);
+    }
+    __syncthreads();
+  }
+
+  // dQ^T tile tt: this lane's column is its query; register r = feature 32*tt + 8*(r/4) + 4g + (r%4)
+  half_t* o1 = p.dq1 + qrow * D;
+  half_t* o2 = p.dq2 + qrow * D;
+#pragma unroll
+  for (int tt = 0; tt < NDT; ++tt)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      h4 v1, v2;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v1[e] = (half_t)(dq1[tt][4 * r4 + e] * p.sm_scale);
+        v2[e] = (half_t)(dq2[tt][4 * r4 + e] * p.sm_scale);
+      }
+      *reinterpret_cast<h4*>(o1 + 32 * tt + 8 * r4 + 4 * g) = v1;
+      *reinterpret_cast<h4*>(o2 + 32 * tt + 8 * r4 + 4 * g) = v2;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+template <int D>
+static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
+  const int n_prep = bwd_num_partials(p.BH, p.N, D);
+  if (p.rms_norm)
+    hipLaunchKernelGGL((bwd_prep_kernel<D, true>), dim3(n_prep), dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((bwd_prep_kernel<D, false>), dim3(n_prep), dim3(256), 0, stream, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(bwd_dlambda_kernel, dim3(1), dim3(256), 0, stream, p.dlam_part, n_prep, p.dlambda);
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+  hipLaunchKernelGGL((bwd_dkdv_kernel<D>), dim3(p.BH * (p.N / DkvCfg<D>::BK)), dim3(256), 0, stream, p);
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+  hipLaunchKernelGGL((bwd_dq_kernel<D>), dim3(p.BH * (p.N / DqCfg<D>::BM)), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_bwd(const BwdParams& p, int D, hipStream_t stream) {
+  switch (D) {
+    case 32:  return launch_bwd_t<32>(p, stream);
+    case 64:  return launch_bwd_t<64>(p, stream);
+    case 128: return launch_bwd_t<128>(p, stream);
+    default:  return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace da

@@ -1,0 +1,100 @@
+// Shared device helpers for the gfx950 differential-attention kernels.
+//
+// MFMA register layouts used throughout (wave64, verified on hardware):
+//   v_mfma_f32_32x32x16_f16  D[32x32] += A[32x16] * B[16x32]
+//     A operand: lane l holds row (l % 32), k = 8*(l / 32) .. +7   (8 halfs = 4 VGPRs)
+//     B operand: lane l holds col (l % 32), k = 8*(l / 32) .. +7
+//     C/D      : lane l holds col (l % 32); register r (0..15) is row 8*(r/4) + 4*(l/32) + (r%4)
+//   ds_read_b64_tr_b16: inside each block of 16 lanes, lane n supplies the address of 4 consecutive
+//     halfs of "row n/4, column chunk n%4"; lane n receives element n of rows 0..3 (a 4x16
+//     transpose), i.e. result[j] = data of lane (4*j + n/4), element (n % 4).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace da {
+
+typedef _Float16 half_t;
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef __fp16 tr4 __attribute__((vector_size(8)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kEps = 1e-5f;
+
+#define DA_LDS __attribute__((address_space(3)))
+
+__device__ __forceinline__ f16v mfma32(h8 a, h8 b, f16v c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// v_permlane32_swap exchanges the upper half of its first register with the lower half of its
+// second one.  Fed the same value in two DISTINCT registers it leaves (lower-half value,
+// upper-half value) of the lane pair (l, l^32) in every lane.  The empty asm keeps the compiler
+// from merging the two copies into one register, which would turn the swap into a self-swap.
+struct LanePair { float lo, hi; };
+__device__ __forceinline__ LanePair lane_pair(float x) {
+  unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+  asm volatile("" : "+v"(b));
+  auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  LanePair p;
+  p.lo = __builtin_bit_cast(float, (unsigned)r[0]);
+  p.hi = __builtin_bit_cast(float, (unsigned)r[1]);
+  return p;
+}
+__device__ __forceinline__ float pair_max(float x) { LanePair p = lane_pair(x); return fmaxf(p.lo, p.hi); }
+__device__ __forceinline__ float pair_sum(float x) { LanePair p = lane_pair(x); return p.lo + p.hi; }
+
+// 4x16 transposing LDS read (see header comment); p must be 8-byte aligned.
+__device__ __forceinline__ h4 lds_read_tr(const half_t* p) {
+  tr4 v = __builtin_amdgcn_ds_read_tr16_b64_v4f16((DA_LDS tr4*)(p));
+  return __builtin_bit_cast(h4, v);
+}
+
+__device__ __forceinline__ h8 join(h4 lo, h4 hi) {
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Cooperative copy of a dense [ROWS x COLS] fp16 tile (row stride COLS in global memory) into an
+// LDS tile with row stride STRIDE, staged through registers so the global loads of the next tile
+// can be in flight while the current one is consumed.
+template <int ROWS, int COLS, int STRIDE, int NT>
+struct TileStage {
+  static constexpr int CPR = COLS / 8;           // 16-byte chunks per row
+  static constexpr int NCH = ROWS * CPR;
+  static constexpr int PER = (NCH + NT - 1) / NT;
+  uint4 reg[PER];
+  __device__ __forceinline__ void load(const half_t* __restrict__ g, int tid) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      int c = tid + i * NT;
+      if (NCH % NT == 0 || c < NCH) reg[i] = *reinterpret_cast<const uint4*>(g + (size_t)c * 8);
+    }
+  }
+  __device__ __forceinline__ void store(half_t* s, int tid) const {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      int c = tid + i * NT;
+      if (NCH % NT == 0 || c < NCH) {
+        int row = c / CPR, col = c % CPR;
+        *reinterpret_cast<uint4*>(s + row * STRIDE + col * 8) = reg[i];
+      }
+    }
+  }
+};
+
+// Workgroup id -> logical tile id such that consecutive logical ids land on the same XCD
+// (workgroups are dealt round-robin to the 8 XCDs, each with a private L2).
+__device__ __forceinline__ int xcd_remap(int wg, int total) {
+  constexpr int kXcd = 8;
+  if (total % kXcd != 0) return wg;
+  return (wg % kXcd) * (total / kXcd) + wg / kXcd;
+}
+
+}  // namespace da

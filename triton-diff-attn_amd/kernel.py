@@ -1,0 +1,117 @@
+"""Autograd wiring of the MI355X differential-attention kernels.
+
+Host-side counterpart of the reference's `_diff_attention` (src/kernel.py:461-575): same class
+name, same `apply` argument order, same 9-slot gradient tuple.  The work itself is done by the
+hand-written HIP kernels in libdiffattn.so, reached through its C ABI; if the library is missing
+the call raises -- there is no other path.
+"""
+import torch
+
+import _native
+
+_SUPPORTED_D = (32, 64, 128)
+_SEQ_MULTIPLE = 128
+
+
+def _check_inputs(Q1, Q2, K1, K2, V):
+    names = ("q1", "q2", "k1", "k2", "v")
+    for n, t in zip(names, (Q1, Q2, K1, K2, V)):
+        if not torch.is_tensor(t):
+            raise TypeError("%s must be a tensor" % n)
+        if t.dtype != torch.float16:
+            raise TypeError("%s must be float16 (got %s); the kernels are fp16-only like the reference "
+                            "(src/kernel.py:3-4)" % (n, t.dtype))
+        if t.dim() != 4:
+            raise ValueError("%s must be [B,H,N,D] (got %d dims)" % (n, t.dim()))
+        if not t.is_cuda:
+            raise ValueError("%s must live on the GPU" % n)
+        if t.device != Q1.device:
+            raise ValueError("all inputs must be on the same device")
+    B, H, N, D = Q1.shape
+    for n, t in zip(names[1:4], (Q2, K1, K2)):
+        if tuple(t.shape) != (B, H, N, D):
+            raise ValueError("%s has shape %s, expected %s" % (n, tuple(t.shape), (B, H, N, D)))
+    if tuple(V.shape) != (B, H, N, 2 * D):
+        raise ValueError("v has shape %s, expected %s" % (tuple(V.shape), (B, H, N, 2 * D)))
+    if D not in _SUPPORTED_D:
+        raise ValueError("head dim %d unsupported; supported: %s" % (D, _SUPPORTED_D))
+    if N % _SEQ_MULTIPLE != 0:
+        raise ValueError("sequence length %d must be a multiple of %d" % (N, _SEQ_MULTIPLE))
+    return B, H, N, D
+
+
+def _lambda_tensor(lambda_scale, device):
+    """The kernels read lambda from device memory (src/kernel.py:138).  A python number is wrapped
+    (a superset of the reference, whose float default cannot reach its kernel)."""
+    if torch.is_tensor(lambda_scale):
+        if lambda_scale.numel() != 1:
+            raise ValueError("lambda_scale must have exactly one element")
+        return lambda_scale.detach().to(device=device, dtype=torch.float16).reshape(1).contiguous()
+    return torch.tensor([float(lambda_scale)], dtype=torch.float16, device=device)
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+class _diff_attention(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, Q1, Q2, K1, K2, V, SM_SCALE, LAMBDA_SCALE, LAMBDA_INIT, rms_norm=False):
+        B, H, N, D = _check_inputs(Q1, Q2, K1, K2, V)
+        lib = _native.lib()
+        dev = Q1.device
+        q1, q2, k1, k2, v = (t.contiguous() for t in (Q1, Q2, K1, K2, V))
+        lam = _lambda_tensor(LAMBDA_SCALE, dev)
+        rms_norm = bool(rms_norm)
+
+        y = torch.empty_like(v)
+        u2 = torch.empty_like(v)
+        lse1 = torch.empty((B, H, N), device=dev, dtype=torch.float32)
+        lse2 = torch.empty((B, H, N), device=dev, dtype=torch.float32)
+        rinv = torch.empty((B, H, N), device=dev, dtype=torch.float32) if rms_norm else None
+
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream().cuda_stream
+            _native.check(lib.diffattn_forward(
+                q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
+                lam.data_ptr(), y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv),
+                B, H, N, D, float(SM_SCALE), float(LAMBDA_INIT), int(rms_norm), stream))
+
+        ctx.save_for_backward(q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam)
+        ctx.SM_SCALE = float(SM_SCALE)
+        ctx.LAMBDA_INIT = float(LAMBDA_INIT)
+        ctx.RMS_NORM = rms_norm
+        ctx.lambda_meta = (LAMBDA_SCALE.dtype, LAMBDA_SCALE.shape) if torch.is_tensor(LAMBDA_SCALE) else None
+        return y
+
+    @staticmethod
+    def backward(ctx, dO):
+        q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam = ctx.saved_tensors
+        B, H, N, D = q1.shape
+        lib = _native.lib()
+        dev = q1.device
+        dO = dO.contiguous()
+        if dO.dtype != torch.float16:
+            dO = dO.to(torch.float16)
+
+        dq1, dq2 = torch.empty_like(q1), torch.empty_like(q2)
+        dk1, dk2 = torch.empty_like(k1), torch.empty_like(k2)
+        dv = torch.empty_like(v)
+        dlam = torch.empty(1, device=dev, dtype=torch.float16)
+        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D)
+        ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream().cuda_stream
+            _native.check(lib.diffattn_backward(
+                q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
+                y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv), dO.data_ptr(),
+                dq1.data_ptr(), dq2.data_ptr(), dk1.data_ptr(), dk2.data_ptr(), dv.data_ptr(), dlam.data_ptr(),
+                ws.data_ptr(), ws_bytes, B, H, N, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, int(ctx.RMS_NORM), stream))
+
+        dlambda = None
+        if ctx.lambda_meta is not None and ctx.needs_input_grad[6]:
+            dtype, shape = ctx.lambda_meta
+            dlambda = dlam.to(dtype).reshape(shape)
+        return dq1, dq2, dk1, dk2, dv, None, dlambda, None, None
