@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Headline benchmark: forward+backward differential attention on one MI355X.
+
+A step is one forward + one backward of `layers.MultiheadDiffAttnKernel` at B=4, H=32, N=2048,
+D=64 (fp16, rms_norm on, lambda 0.5, lambda_init 0.8) on seeded synthetic N(0,1) inputs that are
+resident in HBM before the timed region.  Prints ONE JSON line.
+
+  value       fwd+bwd TFLOP/s, algorithmic matmul FLOPs = 32*B*H*N^2*D per step
+              (forward 12*B*H*N^2*D, backward 20*B*H*N^2*D; 2 FLOP per MAC, softmax not counted)
+  roofline    the dominant kernel (dK/dV backward) against the fp16 dense MFMA peak, timed with
+              events on the launch stream
+  cpu_baseline  the fp32 oracle (forward + autograd backward) on a few (batch, head) units of the
+              same workload on the host cores, scaled to the same FLOP count
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "triton-diff-attn_amd"))
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_FP16_TFLOPS = 2500.0     # MI355X published dense fp16 MFMA peak (2.5 PFLOP/s)
+
+WORKLOADS = {
+    "headline": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0),
+    "config1": dict(B=2, H=16, N=512, D=32, lam=0.5, lambda_init=0.8, rms=True, seed=0, scale=1.0),
+    "config4": dict(B=8, H=32, N=4096, D=128, lam=0.8, lambda_init=0.2, rms=False, seed=4, scale=1.0),
+}
+
+
+def flops(cfg):
+    unit = cfg["B"] * cfg["H"] * cfg["N"] ** 2 * cfg["D"]
+    return 12 * unit, 20 * unit
+
+
+def event_time(fn, iters, torch):
+    """Average milliseconds per call of fn over `iters` calls, measured with events on the current stream."""
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def cpu_baseline(cfg, torch, budget_s=12.0):
+    """Times the fp32 oracle (forward + autograd backward) on a few (b,h) units of the workload."""
+    from oracle import diff_attn_oracle as orc
+    from util import make_inputs
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    N, D = cfg["N"], cfg["D"]
+    units = 8
+    q1, q2, k1, k2, v, dy = make_inputs(1, units, N, D, cfg["seed"], cfg["scale"])
+    lam = torch.tensor([cfg["lam"]], dtype=torch.float16)
+    run = lambda: orc.forward_backward(q1, q2, k1, k2, v, lam, dy, cfg["lambda_init"], cfg["rms"], chunk=1)
+    run()  # warm-up
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        run()
+        reps += 1
+        if time.perf_counter() - t0 > budget_s or reps >= 200:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    fl = 32.0 * units * N * N * D
+    return {
+        "value": fl / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": "%d of %d (batch,head) units of the workload, fp32 oracle forward+autograd backward, %d repetitions, "
+                  "%.3f s per repetition" % (units, cfg["B"] * cfg["H"], reps, dt),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    import _native
+    from layers import MultiheadDiffAttnKernel
+    from util import make_inputs
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    cfg = WORKLOADS[args.workload]
+    B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
+    dev = torch.device("cuda:0")
+    prop = torch.cuda.get_device_properties(0)
+    lib = _native.lib()
+
+    q1, q2, k1, k2, v, dy = (t.to(dev) for t in make_inputs(B, H, N, D, cfg["seed"], cfg["scale"]))
+    leaves = [t.requires_grad_(True) for t in (q1, q2, k1, k2, v)]
+    lam = torch.tensor([cfg["lam"]], dtype=torch.float16, device=dev, requires_grad=True)
+
+    def step():
+        for t in leaves:
+            t.grad = None
+        lam.grad = None
+        y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"])
+        y.backward(dy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms_events = event_time(step, args.steps, torch)
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = max(ms_events, wall_ms)
+
+    f_fwd, f_bwd = flops(cfg)
+    value = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-kernel timings through the C ABI, events on the launch stream ----
+    with torch.no_grad():
+        yb = torch.empty_like(v); u2 = torch.empty_like(v)
+        lse1 = torch.empty(B, H, N, device=dev); lse2 = torch.empty(B, H, N, device=dev)
+        rinv = torch.empty(B, H, N, device=dev)
+        grads = [torch.empty_like(t) for t in (q1, q2, k1, k2, v)]
+        dlam = torch.empty(1, dtype=torch.float16, device=dev)
+        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        stream = torch.cuda.current_stream().cuda_stream
+        sm = 1 / math.sqrt(D)
+
+        def fwd_only():
+            _native.check(lib.diffattn_forward(
+                q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
+                yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(),
+                B, H, N, D, sm, cfg["lambda_init"], int(cfg["rms"]), stream))
+
+        def bwd_stage(mask):
+            return lambda: _native.check(lib.diffattn_backward_stages(
+                q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
+                yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(), dy.data_ptr(),
+                *[g.data_ptr() for g in grads], dlam.data_ptr(), ws.data_ptr(), ws_bytes,
+                B, H, N, D, sm, cfg["lambda_init"], int(cfg["rms"]), mask, stream))
+
+        fwd_only(); bwd_stage(15)()
+        k_iters = max(5, min(args.steps, 30))
+        kernels_ms = {
+            "fwd_kernel": event_time(fwd_only, k_iters, torch),
+            "bwd_prep_kernel": event_time(bwd_stage(1), k_iters, torch),
+            "bwd_dlambda_kernel": event_time(bwd_stage(2), k_iters, torch),
+            "bwd_dkdv_kernel": event_time(bwd_stage(4), k_iters, torch),
+            "bwd_dq_kernel": event_time(bwd_stage(8), k_iters, torch),
+        }
+    unit = B * H * N * N * D
+    dkdv_flops = 16 * unit      # S1,S2 (4) + dP (4) + dV (4) + dK1,dK2 (4), times B*H*N^2*D
+    dkdv_tflops = dkdv_flops / (kernels_ms["bwd_dkdv_kernel"] * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma", "kernel": "bwd_dkdv_kernel", "achieved": dkdv_tflops, "peak": PEAK_FP16_TFLOPS,
+        "unit": "TFLOP/s", "frac": dkdv_tflops / PEAK_FP16_TFLOPS, "traffic": None,
+        "flops_per_launch": dkdv_flops, "ms_per_launch": kernels_ms["bwd_dkdv_kernel"],
+    }
+
+    out = {
+        "metric": "fwd+bwd TFLOP/s & % fp16 MFMA peak, diff-attn B4 H32 N2048 D64",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "%s: diff-attn fwd+bwd B%d H%d N%d D%d fp16 rms_norm=%s lambda=%.1f lambda_init=%.1f"
+                               % (args.workload, B, H, N, D, cfg["rms"], cfg["lam"], cfg["lambda_init"])},
+        "frac_of_fp16_mfma_peak": value / PEAK_FP16_TFLOPS,
+        "fwd_tflops": f_fwd / (kernels_ms["fwd_kernel"] * 1e-3) / 1e12,
+        "bwd_tflops": f_bwd / (sum(kernels_ms[k] for k in kernels_ms if k.startswith("bwd")) * 1e-3) / 1e12,
+        "kernels_ms": kernels_ms,
+        "device": {"name": prop.name, "cus": prop.multi_processor_count,
+                   "clock_mhz": getattr(prop, "clock_rate", 0) / 1e3, "peak_fp16_tflops_used": PEAK_FP16_TFLOPS},
+        "roofline": roofline,
+    }
+    if args.workload != "headline":
+        out["metric"] = "fwd+bwd TFLOP/s & % fp16 MFMA peak, diff-attn"
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, torch)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -77,6 +77,29 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
                       int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
                       void* stream);
 
+/*
+ * Backward, restricted to some of its stream-ordered stages.  No counterpart in the reference
+ * (whose backward is one fused launch); it exists so that a benchmark can time each kernel of
+ * the backward with events on `stream`.  Stage bits, in execution order:
+ *   DIFFATTN_STAGE_PREP    row preprocess: dX, row statistics, d(lambda) partials -> workspace
+ *   DIFFATTN_STAGE_DLAMBDA fixed-order reduction of the partials -> dlambda
+ *   DIFFATTN_STAGE_DKDV    dK1, dK2, dV   (reads the workspace written by PREP)
+ *   DIFFATTN_STAGE_DQ      dQ1, dQ2       (reads the workspace written by PREP)
+ * diffattn_backward(...) == diffattn_backward_stages(..., DIFFATTN_STAGE_ALL, stream).
+ */
+#define DIFFATTN_STAGE_PREP 1u
+#define DIFFATTN_STAGE_DLAMBDA 2u
+#define DIFFATTN_STAGE_DKDV 4u
+#define DIFFATTN_STAGE_DQ 8u
+#define DIFFATTN_STAGE_ALL 15u
+int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                             const void* lambda_scale, const void* y, const void* u2,
+                             const float* lse1, const float* lse2, const float* rinv, const void* dy,
+                             void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
+                             void* workspace, size_t workspace_bytes,
+                             int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                             unsigned stage_mask, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

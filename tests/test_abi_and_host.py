@@ -1,0 +1,90 @@
+"""CPU-only checks: the C-ABI library loads and exports every symbol include/diffattn.h declares,
+argument rejection works without a GPU, and the host wrappers validate their inputs."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "diffattn.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(diffattn_[a-z_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    assert declared_symbols() == sorted([
+        "diffattn_abi_version", "diffattn_strerror", "diffattn_forward",
+        "diffattn_backward_workspace_bytes", "diffattn_backward", "diffattn_backward_stages"])
+
+
+def test_library_exports_every_declared_symbol():
+    import _native
+    lib = _native.lib()
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+        assert name in _native.SYMBOLS, "binding table misses %s" % name
+    assert lib.diffattn_abi_version() == 1
+
+
+def test_argument_rejection_needs_no_gpu():
+    import _native
+    lib = _native.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf) & ~255
+    p += 256
+    args = lambda B, H, N, D: ([p] * 5 + [p, p, p, p, p, p] + [B, H, N, D, 0.125, 0.8, 1, None])
+    assert lib.diffattn_forward(*([None] + args(1, 1, 128, 64)[1:])) == -1
+    assert lib.diffattn_forward(*args(1, 1, 128, 48)) == -2
+    assert lib.diffattn_forward(*args(0, 1, 128, 64)) == -2
+    assert lib.diffattn_forward(*args(1, 1, 100, 64)) == -3
+    bad = args(1, 1, 128, 64)
+    bad[0] = p + 2
+    assert lib.diffattn_forward(*bad) == -5
+    assert lib.diffattn_backward_workspace_bytes(1, 1, 100, 64) == 0
+    assert lib.diffattn_backward_workspace_bytes(1, 1, 128, 48) == 0
+    need = lib.diffattn_backward_workspace_bytes(2, 3, 256, 64)
+    rows = 2 * 3 * 256
+    assert need >= rows * 128 * 2 + 4 * rows * 4
+    bargs = [p] * 5 + [p, p, p, p, p, p, p] + [p] * 6 + [p, need - 1, 2, 3, 256, 64, 0.125, 0.8, 1, None]
+    assert lib.diffattn_backward(*bargs) == -4
+    for code in (0, -1, -2, -3, -4, -5):
+        assert len(lib.diffattn_strerror(code)) > 0
+
+
+def test_host_validation_errors():
+    from kernel import _check_inputs, _lambda_tensor
+
+    class FakeCuda(torch.Tensor):
+        pass
+
+    t = lambda *s, dt=torch.float16: torch.zeros(*s, dtype=dt)
+    with pytest.raises(TypeError):
+        _check_inputs(t(1, 1, 128, 64, dt=torch.float32), *[t(1, 1, 128, 64)] * 3, t(1, 1, 128, 128))
+    with pytest.raises(ValueError):
+        _check_inputs(t(1, 128, 64), *[t(1, 1, 128, 64)] * 3, t(1, 1, 128, 128))
+    with pytest.raises(ValueError):  # CPU tensors are rejected: there is no CPU path
+        _check_inputs(*[t(1, 1, 128, 64)] * 4, t(1, 1, 128, 128))
+    with pytest.raises(ValueError):
+        _lambda_tensor(torch.zeros(2), torch.device("cpu"))
+    lam = _lambda_tensor(0.25, torch.device("cpu"))
+    assert lam.dtype == torch.float16 and lam.shape == (1,) and lam.item() == 0.25
+
+
+def test_drop_in_signature_matches_reference():
+    import inspect
+    import layers
+    from kernel import _diff_attention
+    sig = inspect.signature(layers.MultiheadDiffAttnKernel)
+    assert list(sig.parameters) == ["q1", "q2", "k1", "k2", "v", "lambda_scale", "lambda_init", "rms_norm"]
+    assert sig.parameters["lambda_scale"].default == -0.5
+    assert sig.parameters["lambda_init"].default == 0.8
+    assert sig.parameters["rms_norm"].default is False
+    fsig = inspect.signature(_diff_attention.forward)
+    assert list(fsig.parameters) == ["ctx", "Q1", "Q2", "K1", "K2", "V", "SM_SCALE", "LAMBDA_SCALE", "LAMBDA_INIT", "rms_norm"]
+    assert issubclass(_diff_attention, torch.autograd.Function)

@@ -76,13 +76,13 @@ size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D) {
   return ws_layout(B * H, N, D).total;
 }
 
-int diffattn_backward(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
-                      const void* lambda_scale, const void* y, const void* u2,
-                      const float* lse1, const float* lse2, const float* rinv, const void* dy,
-                      void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
-                      void* workspace, size_t workspace_bytes,
-                      int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
-                      void* stream) {
+int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                             const void* lambda_scale, const void* y, const void* u2,
+                             const float* lse1, const float* lse2, const float* rinv, const void* dy,
+                             void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
+                             void* workspace, size_t workspace_bytes,
+                             int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                             unsigned stage_mask, void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy ||
       !dq1 || !dq2 || !dk1 || !dk2 || !dv || !dlambda || !workspace)
     return DIFFATTN_EINVAL_NULL;
@@ -104,7 +104,20 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
   p.dx = (half_t*)(ws + w.dx); p.stat = (float*)(ws + w.stat);
   p.dlam_part = (float*)(ws + w.part); p.n_part = bwd_num_partials(B * H, N, D);
   p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = rms_norm ? 1 : 0;
+  p.stages = stage_mask & DIFFATTN_STAGE_ALL;
   return (int)launch_bwd(p, D, (hipStream_t)stream);
+}
+
+int diffattn_backward(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                      const void* lambda_scale, const void* y, const void* u2,
+                      const float* lse1, const float* lse2, const float* rinv, const void* dy,
+                      void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
+                      void* workspace, size_t workspace_bytes,
+                      int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                      void* stream) {
+  return diffattn_backward_stages(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy,
+                                  dq1, dq2, dk1, dk2, dv, dlambda, workspace, workspace_bytes,
+                                  B, H, N, D, sm_scale, lambda_init, rms_norm, DIFFATTN_STAGE_ALL, stream);
 }
 
 }  // extern "C"

@@ -451,18 +451,27 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(BwdParams p) {
 template <int D>
 static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
   const int n_prep = bwd_num_partials(p.BH, p.N, D);
-  if (p.rms_norm)
-    hipLaunchKernelGGL((bwd_prep_kernel<D, true>), dim3(n_prep), dim3(256), 0, stream, p);
-  else
-    hipLaunchKernelGGL((bwd_prep_kernel<D, false>), dim3(n_prep), dim3(256), 0, stream, p);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(bwd_dlambda_kernel, dim3(1), dim3(256), 0, stream, p.dlam_part, n_prep, p.dlambda);
-  if ((e = hipGetLastError()) != hipSuccess) return e;
-  hipLaunchKernelGGL((bwd_dkdv_kernel<D>), dim3(p.BH * (p.N / DkvCfg<D>::BK)), dim3(256), 0, stream, p);
-  if ((e = hipGetLastError()) != hipSuccess) return e;
-  hipLaunchKernelGGL((bwd_dq_kernel<D>), dim3(p.BH * (p.N / DqCfg<D>::BM)), dim3(256), 0, stream, p);
-  return hipGetLastError();
+  hipError_t e = hipSuccess;
+  if (p.stages & 1u) {
+    if (p.rms_norm)
+      hipLaunchKernelGGL((bwd_prep_kernel<D, true>), dim3(n_prep), dim3(256), 0, stream, p);
+    else
+      hipLaunchKernelGGL((bwd_prep_kernel<D, false>), dim3(n_prep), dim3(256), 0, stream, p);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+  }
+  if (p.stages & 2u) {
+    hipLaunchKernelGGL(bwd_dlambda_kernel, dim3(1), dim3(256), 0, stream, p.dlam_part, n_prep, p.dlambda);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+  }
+  if (p.stages & 4u) {
+    hipLaunchKernelGGL((bwd_dkdv_kernel<D>), dim3(p.BH * (p.N / DkvCfg<D>::BK)), dim3(256), 0, stream, p);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+  }
+  if (p.stages & 8u) {
+    hipLaunchKernelGGL((bwd_dq_kernel<D>), dim3(p.BH * (p.N / DqCfg<D>::BM)), dim3(256), 0, stream, p);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+  }
+  return e;
 }
 
 hipError_t launch_bwd(const BwdParams& p, int D, hipStream_t stream) {

@@ -33,6 +33,7 @@ struct BwdParams {
   int BH, N;
   float sm_scale, lambda_init;
   int rms_norm;
+  unsigned stages;              // bit 0 row preprocess, 1 d(lambda) reduce, 2 dK/dV, 3 dQ
 };
 
 hipError_t launch_fwd(const FwdParams& p, int D, hipStream_t stream);
