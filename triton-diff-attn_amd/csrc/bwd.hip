@@ -125,7 +125,7 @@ struct DkvCfg {
 };
 
 template <int D>
-__global__ __launch_bounds__(256) void bwd_dkdv_kernel(BwdParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_kernel(BwdParams p) {
   using C = DkvCfg<D>;
   constexpr int DV = C::DV, NT = C::NT, BK = C::BK, BQ = C::BQ, QS = C::QS, XS = C::XS;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32, NVT = DV / 32;
@@ -210,8 +210,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(BwdParams p) {
     const half_t* sQ2 = sQ1 + C::Q_TILE;
     const half_t* sX = sQ1 + 2 * C::Q_TILE;
     const float* sStat = reinterpret_cast<const float*>(sQ1 + 2 * C::Q_TILE + C::X_TILE);
-    const bool more = (qt + 1 < n_qt);
-    if (more) stage_load(qt + 1);
+    stage_load((qt + 1 < n_qt) ? qt + 1 : qt);   // the last iteration re-reads its own tile: harmless
 
 #pragma unroll
     for (int qs = 0; qs < BQ / 32; ++qs) {
@@ -272,7 +271,7 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(BwdParams p) {
       }
     }
 
-    if (more) stage_store((qt + 1) & 1);
+    stage_store((qt + 1) & 1);
     __syncthreads();
   }
 
@@ -310,7 +309,7 @@ struct DqCfg {
 };
 
 template <int D>
-__global__ __launch_bounds__(256) void bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<D>;
   constexpr int DV = C::DV, NT = C::NT, BM = C::BM, BN = C::BN, KS = C::KS, VS = C::VS;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
@@ -374,12 +373,10 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(BwdParams p) {
     const half_t* sK1 = smem + (t & 1) * C::STAGE;
     const half_t* sK2 = sK1 + C::K_TILE;
     const half_t* sV = sK1 + 2 * C::K_TILE;
-    const bool more = (t + 1 < n_tiles);
-    if (more) {
-      stK1.load(gk1 + (size_t)(t + 1) * BN * D, tid);
-      stK2.load(gk2 + (size_t)(t + 1) * BN * D, tid);
-      stV.load(gv + (size_t)(t + 1) * BN * DV, tid);
-    }
+    const int tn = (t + 1 < n_tiles) ? t + 1 : t;   // the last iteration re-reads its own tile: harmless
+    stK1.load(gk1 + (size_t)tn * BN * D, tid);
+    stK2.load(gk2 + (size_t)tn * BN * D, tid);
+    stV.load(gv + (size_t)tn * BN * DV, tid);
 
 #pragma unroll
     for (int ksub = 0; ksub < BN / 32; ++ksub) {
@@ -422,7 +419,7 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(BwdParams p) {
       }
     }
 
-    if (more) {
+    {
       half_t* nb = smem + ((t + 1) & 1) * C::STAGE;
       stK1.store(nb, tid); stK2.store(nb + C::K_TILE, tid); stV.store(nb + 2 * C::K_TILE, tid);
     }

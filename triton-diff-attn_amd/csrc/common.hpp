@@ -21,6 +21,7 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef float f4v __attribute__((ext_vector_type(4)));
 typedef __fp16 tr4 __attribute__((vector_size(8)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -69,12 +70,12 @@ struct TileStage {
   static constexpr int CPR = COLS / 8;           // 16-byte chunks per row
   static constexpr int NCH = ROWS * CPR;
   static constexpr int PER = (NCH + NT - 1) / NT;
-  uint4 reg[PER];
+  u32x4 reg[PER];
   __device__ __forceinline__ void load(const half_t* __restrict__ g, int tid) {
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       int c = tid + i * NT;
-      if (NCH % NT == 0 || c < NCH) reg[i] = *reinterpret_cast<const uint4*>(g + (size_t)c * 8);
+      if (NCH % NT == 0 || c < NCH) reg[i] = *reinterpret_cast<const u32x4*>(g + (size_t)c * 8);
     }
   }
   __device__ __forceinline__ void store(half_t* s, int tid) const {
@@ -83,7 +84,7 @@ struct TileStage {
       int c = tid + i * NT;
       if (NCH % NT == 0 || c < NCH) {
         int row = c / CPR, col = c % CPR;
-        *reinterpret_cast<uint4*>(s + row * STRIDE + col * 8) = reg[i];
+        *reinterpret_cast<u32x4*>(s + row * STRIDE + col * 8) = reg[i];
       }
     }
   }

@@ -32,7 +32,7 @@ struct FwdCfg {
 };
 
 template <int D, bool RMS>
-__global__ __launch_bounds__(512) void fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fwd_kernel(FwdParams p) {
   using C = FwdCfg<D>;
   constexpr int DV = C::DV, BN = C::BN, KS = C::KS, VS = C::VS, NT = C::NT, BM = C::BM;
   constexpr int NKS = D / 16;                // k-steps of the score product
@@ -89,12 +89,11 @@ __global__ __launch_bounds__(512) void fwd_kernel(FwdParams p) {
   for (int t = 0; t < n_tiles; ++t) {
     const half_t* sK = smem + (t & 1) * C::STAGE + k_off;
     const half_t* sV = smem + (t & 1) * C::STAGE + v_off;
-    const bool more = (t + 1 < n_tiles);
-    if (more) {
-      stK1.load(gk1 + (size_t)(t + 1) * BN * D, tid);
-      stK2.load(gk2 + (size_t)(t + 1) * BN * D, tid);
-      stV.load(gv + (size_t)(t + 1) * BN * DV, tid);
-    }
+    // prefetch the next tile into registers (the last iteration re-reads its own tile: harmless)
+    const int tn = (t + 1 < n_tiles) ? t + 1 : t;
+    stK1.load(gk1 + (size_t)tn * BN * D, tid);
+    stK2.load(gk2 + (size_t)tn * BN * D, tid);
+    stV.load(gv + (size_t)tn * BN * DV, tid);
 
     f16v s[NKT];
 #pragma unroll
@@ -144,7 +143,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(FwdParams p) {
       }
     }
 
-    if (more) {
+    {
       half_t* nb = smem + ((t + 1) & 1) * C::STAGE;
       stK1.store(nb, tid); stK2.store(nb + C::K_TILE, tid); stV.store(nb + 2 * C::K_TILE, tid);
     }
