@@ -15,6 +15,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed-fp32 VALU instructions are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-fno-honor-nans",
     "-Wno-unused-command-line-argument",
 ]
 

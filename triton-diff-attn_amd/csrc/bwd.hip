@@ -309,7 +309,7 @@ struct DqCfg {
 };
 
 template <int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<D>;
   constexpr int DV = C::DV, NT = C::NT, BM = C::BM, BN = C::BN, KS = C::KS, VS = C::VS;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;

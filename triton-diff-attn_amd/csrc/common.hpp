@@ -62,6 +62,73 @@ __device__ __forceinline__ h8 join(h4 lo, h4 hi) {
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+#define DA_GLOBAL __attribute__((address_space(1)))
+
+// ---- LDS tiles: dense rows, 16-byte chunks XOR-swizzled inside each row ------------------------
+// A tile row of COLS halfs is CPR = COLS/8 chunks of 16 bytes; chunk c of row r is stored at chunk
+// position c ^ swz_f<CPR>(r).  The functions are chosen so that both access patterns of the
+// kernels hit every LDS bank once: (a) 16 consecutive rows reading the same chunk with 128-bit
+// loads, (b) the transposing read, where 32 lanes read 4 consecutive rows x 4 consecutive chunks.
+template <int CPR>
+__device__ __forceinline__ int swz_f(int row) {
+  if constexpr (CPR == 4) {
+    return (row >> 2) & 3;
+  } else if constexpr (CPR == 8) {
+    const int k = (row >> 1) & 7;
+    return ((k & 1) << 2) | (k >> 1);
+  } else {
+    return ((row & 3) << 2) | ((row >> 2) & 3);
+  }
+}
+
+// Offset in halfs of element (row, col) of a swizzled tile with COLS halfs per row.
+template <int COLS>
+__device__ __forceinline__ int swz_off(int row, int col) {
+  constexpr int CPR = COLS / 8;
+  return row * COLS + ((((col >> 3) ^ swz_f<CPR>(row))) << 3) + (col & 7);
+}
+
+// One direct global->LDS load of 16 bytes per lane: lane l's bytes land at lds_base + 16*l, where
+// lds_base must be wave-uniform.  Written as inline assembly so that the compiler's wait-count
+// insertion does not serialise later, unrelated LDS reads behind it; the caller orders it with
+// wait_async_tiles() and a barrier before the data is read.
+__device__ __forceinline__ void async_copy16(const half_t* g, half_t* lds_base) {
+  const unsigned lds_addr = (unsigned)(unsigned long)((DA_LDS char*)lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :: "v"(g), "s"(lds_addr) : "memory");
+}
+
+// Asynchronous copy of a dense [ROWS x COLS] fp16 tile (row stride COLS in global memory) into a
+// swizzled LDS tile with direct global->LDS loads: no registers, no LDS store instructions.  One
+// wave-instruction moves 64 chunks; the hardware writes lane l's 16 bytes at (wave-uniform LDS
+// base) + 16*l, so the swizzle is applied by choosing which global chunk each lane fetches.  NW
+// waves share the tile's instructions round-robin.  Completion: s_waitcnt vmcnt(0), then a barrier.
+template <int ROWS, int COLS, int NW>
+struct AsyncTile {
+  static constexpr int CPR = COLS / 8;
+  static constexpr int NINST = ROWS * CPR / 64;
+  static constexpr int PER = (NINST + NW - 1) / NW;
+  static_assert((ROWS * CPR) % 64 == 0, "tile must be a whole number of 1 KiB pieces");
+  // global offset (halfs) inside the tile of the chunk that `lane` of `wave` fetches in its k-th instruction
+  __device__ static __forceinline__ int goff(int wave, int lane, int k) {
+    const int L = (wave + NW * k) * 64 + lane;
+    const int row = L / CPR, cpos = L % CPR;
+    return row * COLS + ((cpos ^ swz_f<CPR>(row)) << 3);
+  }
+  // issues this wave's instructions k0 .. k1-1 (of PER) for the tile
+  template <int K0 = 0, int K1 = PER>
+  __device__ static __forceinline__ void issue(const half_t* gtile, half_t* lds_tile, int wave, int lane) {
+#pragma unroll
+    for (int k = K0; k < K1; ++k) {
+      const int inst = wave + NW * k;
+      if (NINST % NW == 0 || inst < NINST)
+        async_copy16(gtile + goff(wave, lane, k), lds_tile + inst * 512);
+    }
+  }
+};
+
+__device__ __forceinline__ void wait_async_tiles() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // Cooperative copy of a dense [ROWS x COLS] fp16 tile (row stride COLS in global memory) into an
 // LDS tile with row stride STRIDE, staged through registers so the global loads of the next tile
 // can be in flight while the current one is consumed.

@@ -20,31 +20,38 @@ template <int D>
 struct FwdCfg {
   static constexpr int DV = 2 * D;
   static constexpr int BN = (D <= 64) ? 64 : 32;   // keys per tile
+  static constexpr int QS = 1;                     // 32-row query blocks per wave
   static constexpr int BM = 128;                   // query rows per workgroup
-  static constexpr int NT = 512;                   // threads per workgroup
-  static constexpr int KS = D + 8;                 // K row stride in LDS (halfs), 16 B pad
-  static constexpr int VS = DV + 32;               // V row stride in LDS (halfs), 64 B pad
-  static constexpr int K_TILE = BN * KS;           // halfs
-  static constexpr int V_TILE = BN * VS;
-  static constexpr int STAGE = 2 * K_TILE + V_TILE;
-  static constexpr int XCHG = 4 * (DV / 32) * 16 * 64 * 2;   // halfs needed by the epilogue exchange
-  static constexpr int SMEM = (2 * STAGE > XCHG) ? 2 * STAGE : XCHG;
+  static constexpr int NW = 2 * BM / (32 * QS);    // waves per workgroup: half of them per softmax stream
+  static constexpr int NT = NW * 64;
+  static constexpr int OCC = (QS == 2) ? 1 : 2;    // waves per SIMD the register budget is sized for
+  static constexpr int K_TILE = BN * D;            // halfs, one stream (swizzled, unpadded)
+  static constexpr int V_TILE = BN * DV;
+  static constexpr int K_BUF = 2 * K_TILE;         // K1 and K2 of one tile
+  static constexpr int TILES = 2 * K_BUF + 2 * V_TILE;       // two K buffers and two V buffers
+  static constexpr int XCHG = (BM / 32) * (DV / 32) * 16 * 64 * 2;   // halfs needed by the epilogue exchange
+  static constexpr int SMEM = (TILES > XCHG) ? TILES : XCHG;
 };
 
+constexpr float kRescaleThreshold = 8.0f;   // log2 units: probabilities stay below 2^8 between updates of the row max
+
 template <int D, bool RMS>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void fwd_kernel(FwdParams p) {
+__global__ __launch_bounds__(FwdCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::OCC, FwdCfg<D>::OCC)))
+void fwd_kernel(FwdParams p) {
   using C = FwdCfg<D>;
-  constexpr int DV = C::DV, BN = C::BN, KS = C::KS, VS = C::VS, NT = C::NT, BM = C::BM;
+  constexpr int DV = C::DV, BN = C::BN, NW = C::NW, BM = C::BM, QS = C::QS;
   constexpr int NKS = D / 16;                // k-steps of the score product
   constexpr int NKT = BN / 32;               // 32-key tiles of S^T
   constexpr int NKK = BN / 16;               // k-steps of the P*V product
   constexpr int NOT = DV / 32;               // 32-row tiles of O^T
 
   __shared__ __attribute__((aligned(16))) half_t smem[C::SMEM];
+  half_t* const sKbuf = smem;                       // [2][K1 tile, K2 tile]
+  half_t* const sVbuf = smem + 2 * C::K_BUF;        // [2][V tile]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int st = wave >> 2, qw = wave & 3;   // stream, 32-row block inside the workgroup
+  const int st = wave / (NW / 2), qw = wave % (NW / 2);   // stream, block of 32*QS rows inside the workgroup
   const int j = lane & 31, g = lane >> 5;
 
   const int n_qt = p.N / BM;
@@ -52,160 +59,268 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int bh = tile / n_qt, qt = tile % n_qt;
   const size_t qk_base = (size_t)bh * p.N * D;
   const size_t v_base = (size_t)bh * p.N * DV;
-  const int qrow = qt * BM + qw * 32 + j;
-
-  const float c = p.sm_scale * kLog2e;       // scores are handled in log2 units
+  const int qrow0 = qt * BM + qw * 32 * QS + j;   // this lane's query row of block qs is qrow0 + 32*qs
 
   // Q fragments (B operand): column j = this lane's query, k = 8g..8g+7 of each 16-wide k-step.
-  h8 qf[NKS];
+  // They are pre-multiplied by sm_scale*log2(e), so the MFMA result is the score in log2 units.
+  h8 qf[QS][NKS];
   {
-    const half_t* r = (st ? p.q2 : p.q1) + qk_base + (size_t)qrow * D + 8 * g;
+    const float c = p.sm_scale * kLog2e;
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) qf[ks] = *reinterpret_cast<const h8*>(r + 16 * ks);
+    for (int qs = 0; qs < QS; ++qs) {
+      const half_t* r = (st ? p.q2 : p.q1) + qk_base + (size_t)(qrow0 + 32 * qs) * D + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        h8 q = *reinterpret_cast<const h8*>(r + 16 * ks);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) q[e] = (half_t)((float)q[e] * c);
+        qf[qs][ks] = q;
+      }
+    }
   }
 
-  f16v o[NOT];
+  f16v o[QS][NOT];
 #pragma unroll
-  for (int t = 0; t < NOT; ++t)
+  for (int qs = 0; qs < QS; ++qs)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
-  float m = -INFINITY, l = 0.f;
+    for (int t = 0; t < NOT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[qs][t][r] = 0.f;
+  // The running reference m of the online softmax is folded into the score product as the
+  // initial accumulator value -m, so the MFMA result is already s - m.
+  float m[QS], l[QS];
+  f16v negm[QS];
+#pragma unroll
+  for (int qs = 0; qs < QS; ++qs) {
+    m[qs] = 0.f; l[qs] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) negm[qs][r] = 0.f;
+  }
 
-  TileStage<BN, D, KS, NT> stK1, stK2;
-  TileStage<BN, DV, VS, NT> stV;
+  using KTile = AsyncTile<BN, D, NW>;
+  using VTile = AsyncTile<BN, DV, NW>;
   const half_t* gk1 = p.k1 + qk_base;
   const half_t* gk2 = p.k2 + qk_base;
   const half_t* gv = p.v + v_base;
-
-  stK1.load(gk1, tid); stK2.load(gk2, tid); stV.load(gv, tid);
-  stK1.store(smem, tid); stK2.store(smem + C::K_TILE, tid); stV.store(smem + 2 * C::K_TILE, tid);
-  __syncthreads();
-
-  // per-lane LDS offsets (halfs)
-  const int k_off = st * C::K_TILE + j * KS + 8 * g;                        // K A-fragment
-  const int v_off = 2 * C::K_TILE + (4 * g + ((lane & 15) >> 2)) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-
   const int n_tiles = p.N / BN;
-  for (int t = 0; t < n_tiles; ++t) {
-    const half_t* sK = smem + (t & 1) * C::STAGE + k_off;
-    const half_t* sV = smem + (t & 1) * C::STAGE + v_off;
-    // prefetch the next tile into registers (the last iteration re-reads its own tile: harmless)
-    const int tn = (t + 1 < n_tiles) ? t + 1 : t;
-    stK1.load(gk1 + (size_t)tn * BN * D, tid);
-    stK2.load(gk2 + (size_t)tn * BN * D, tid);
-    stV.load(gv + (size_t)tn * BN * DV, tid);
+  constexpr int VH = (VTile::PER + 1) / 2;   // V instructions are issued in two groups
+  auto load_k1 = [&](int tk, int buf) { KTile::issue(gk1 + (size_t)tk * BN * D, sKbuf + buf * C::K_BUF, wave, lane); };
+  auto load_k2 = [&](int tk, int buf) { KTile::issue(gk2 + (size_t)tk * BN * D, sKbuf + buf * C::K_BUF + C::K_TILE, wave, lane); };
+  auto load_va = [&](int tv, int buf) { VTile::template issue<0, VH>(gv + (size_t)tv * BN * DV, sVbuf + buf * C::V_TILE, wave, lane); };
+  auto load_vb = [&](int tv, int buf) { VTile::template issue<VH, VTile::PER>(gv + (size_t)tv * BN * DV, sVbuf + buf * C::V_TILE, wave, lane); };
 
-    f16v s[NKT];
-#pragma unroll
-    for (int kt = 0; kt < NKT; ++kt) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[kt][r] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        h8 a = *reinterpret_cast<const h8*>(sK + kt * 32 * KS + 16 * ks);
-        s[kt] = mfma32(a, qf[ks], s[kt]);
-      }
-    }
-    float mx = s[0][0];
+  // A-fragments of K for all k-steps of all 32-key tiles: row kt*32 + j, halfs 16ks + 8g .. +7
+  auto read_k = [&](const half_t* sK, h8 (&ka)[NKT][NKS]) {
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kt][r]);
-    mx = pair_max(mx);
-    const float mnew = fmaxf(m, mx * c);
-    const float alpha = fast_exp2(m - mnew);
-    m = mnew;
-    float rs = 0.f;
-    h8 pb[NKK];          // P^T as B operands: pb[kk] covers keys 16kk..16kk+15 (accumulator order)
+      for (int ks = 0; ks < NKS; ++ks)
+        ka[kt][ks] = *reinterpret_cast<const h8*>(sK + swz_off<D>(kt * 32 + j, 16 * ks + 8 * g));
+  };
+  auto scores = [&](const h8 (&ka)[NKT][NKS], f16v (&s)[QS][NKT]) {
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float e = fast_exp2(__builtin_fmaf(s[kt][r], c, -mnew));
-        rs += e;
-        pb[kt * 2 + r / 8][r % 8] = (half_t)e;
+      for (int qs = 0; qs < QS; ++qs) {
+        s[qs][kt] = negm[qs];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) s[qs][kt] = mfma32(ka[kt][ks], qf[qs][ks], s[qs][kt]);
       }
-    l = l * alpha + rs;
-    if (__any(alpha != 1.0f)) {
+  };
+
+  // prologue: K tiles 0 and 1 and V tile 0; scores of tile 0
+  load_k1(0, 0); load_k2(0, 0);
+  load_k1((n_tiles > 1) ? 1 : 0, 1); load_k2((n_tiles > 1) ? 1 : 0, 1);
+  load_va(0, 0); load_vb(0, 0);
+  wait_async_tiles();
+  __syncthreads();
+  f16v s_a[QS][NKT], s_b[QS][NKT];
+  {
+    h8 ka[NKT][NKS];
+    read_k(sKbuf + st * C::K_TILE, ka);
+    scores(ka, s_a);
+  }
+  __syncthreads();   // K buffer 0 is overwritten by the first iteration's prefetch
+
+  // transposing-read coordinates of this lane inside a 16-key k-step: key row and feature column
+  const int tr_row = 4 * g + ((lane & 15) >> 2);
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  // One iteration: softmax of tile t (scores in s_cur) and its P*V product, overlapped with the score
+  // product of tile t+1 (into s_nxt).
+  auto iteration = [&](int t, f16v (&s_cur)[QS][NKT], f16v (&s_nxt)[QS][NKT]) {
+    // Asynchronous prefetch straight into LDS: K tile t+2 replaces K tile t (consumed one iteration
+    // ago), V tile t+1 replaces V tile t-1 (clamped at the end: harmless re-reads).  The groups of
+    // load instructions are spread over the iteration so that the waves do not queue up behind each
+    // other at the memory pipeline.
+    const int tk = (t + 2 < n_tiles) ? t + 2 : n_tiles - 1;
+    const int tv = (t + 1 < n_tiles) ? t + 1 : n_tiles - 1;
+    load_k1(tk, t & 1);
+
+    // K fragments of the next tile are requested first; the row maxima of this tile are reduced
+    // while they arrive.
+    h8 ka[NKT][NKS];
+    read_k(sKbuf + ((t + 1) & 1) * C::K_BUF + st * C::K_TILE, ka);
+
+    float mx[QS];
 #pragma unroll
-      for (int tt = 0; tt < NOT; ++tt)
+    for (int qs = 0; qs < QS; ++qs) {
+      float mx0 = fmaxf(s_cur[qs][0][0], s_cur[qs][0][1]), mx1 = fmaxf(s_cur[qs][0][2], s_cur[qs][0][3]);
+      float mx2 = fmaxf(s_cur[qs][0][4], s_cur[qs][0][5]), mx3 = fmaxf(s_cur[qs][0][6], s_cur[qs][0][7]);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[tt][r] *= alpha;
+      for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+        for (int r = (kt == 0 ? 8 : 0); r < 16; r += 8) {
+          mx0 = fmaxf(mx0, fmaxf(s_cur[qs][kt][r + 0], s_cur[qs][kt][r + 1]));
+          mx1 = fmaxf(mx1, fmaxf(s_cur[qs][kt][r + 2], s_cur[qs][kt][r + 3]));
+          mx2 = fmaxf(mx2, fmaxf(s_cur[qs][kt][r + 4], s_cur[qs][kt][r + 5]));
+          mx3 = fmaxf(mx3, fmaxf(s_cur[qs][kt][r + 6], s_cur[qs][kt][r + 7]));
+        }
+      mx[qs] = fmaxf(fmaxf(mx0, mx1), fmaxf(mx2, mx3));
+    }
+    float mxall = mx[0];
+#pragma unroll
+    for (int qs = 1; qs < QS; ++qs) mxall = fmaxf(mxall, mx[qs]);
+    // The reference only moves when some row of the wave outgrew it by more than the threshold
+    // (always on the first tile, where it starts at 0 with nothing accumulated yet).
+    if (__any(mxall > kRescaleThreshold) || t == 0) {
+#pragma unroll
+      for (int qs = 0; qs < QS; ++qs) {
+        const float pm = pair_max(mx[qs]);
+        const float d = (t == 0) ? pm : fmaxf(pm, 0.f);
+        const float alpha = fast_exp2(-d);
+        m[qs] += d;
+        l[qs] *= alpha;
+#pragma unroll
+        for (int tt = 0; tt < NOT; ++tt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[qs][tt][r] *= alpha;
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) s_cur[qs][kt][r] -= d;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) negm[qs][r] = -m[qs];
+      }
     }
 
+    // From here on one basic block: the score product of the next tile and the P*V product of this
+    // tile run on the matrix unit while the exponentials run on the VALU.
+    load_k2(tk, t & 1);
+    scores(ka, s_nxt);
+
+    h8 pb[QS][NKK];      // P^T as B operands: pb[kk] covers keys 16kk..16kk+15 (accumulator order)
+    const h2 ones = {(half_t)1.0f, (half_t)1.0f};
+#pragma unroll
+    for (int qs = 0; qs < QS; ++qs) {
+      float rs = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          h2 e2;
+          e2[0] = (half_t)fast_exp2(s_cur[qs][kt][r]);
+          e2[1] = (half_t)fast_exp2(s_cur[qs][kt][r + 1]);
+          rs = __builtin_amdgcn_fdot2(e2, ones, rs, false);   // row sum of the rounded probabilities
+          pb[qs][kt * 2 + r / 8][r % 8] = e2[0];
+          pb[qs][kt * 2 + r / 8][r % 8 + 1] = e2[1];
+        }
+      l[qs] += rs;
+    }
+
+    const half_t* sV = sVbuf + (t & 1) * C::V_TILE;
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {
+      if (kk == 0) load_va(tv, (t + 1) & 1);
+      if (kk == NKK / 2) load_vb(tv, (t + 1) & 1);
 #pragma unroll
       for (int tt = 0; tt < NOT; ++tt) {
-        const half_t* vp = sV + (16 * kk) * VS + 32 * tt;
-        h8 a = join(lds_read_tr(vp), lds_read_tr(vp + 8 * VS));
-        o[tt] = mfma32(a, pb[kk], o[tt]);
+        h8 a = join(lds_read_tr(sV + swz_off<DV>(16 * kk + tr_row, 32 * tt + tr_col)),
+                    lds_read_tr(sV + swz_off<DV>(16 * kk + 8 + tr_row, 32 * tt + tr_col)));
+#pragma unroll
+        for (int qs = 0; qs < QS; ++qs) o[qs][tt] = mfma32(a, pb[qs][kk], o[qs][tt]);
       }
     }
 
-    {
-      half_t* nb = smem + ((t + 1) & 1) * C::STAGE;
-      stK1.store(nb, tid); stK2.store(nb + C::K_TILE, tid); stV.store(nb + 2 * C::K_TILE, tid);
-    }
+    wait_async_tiles();
     __syncthreads();
+  };
+
+  // the tile count is even (N is a multiple of 128, tiles are at most 64 keys)
+  for (int t = 0; t < n_tiles; t += 2) {
+    iteration(t, s_a, s_b);
+    iteration(t + 1, s_b, s_a);
   }
 
   // ---- epilogue: every quantity below is per query = per lane pair (l, l^32) ----
-  l = pair_sum(l);
-  const float inv = 1.0f / l;
-  const size_t row = (size_t)bh * p.N + qrow;
-  {
-    float* lse = st ? p.lse2 : p.lse1;
-    if (g == 0 && lse) lse[row] = (m + __builtin_log2f(l)) * kLn2;
-  }
-  // stream-2 waves hand softmax(S2)V to the stream-1 wave that owns the same rows (same lane,
-  // same register index), through the now idle tile memory
-  float* xchg = reinterpret_cast<float*>(smem) + (size_t)qw * NOT * 16 * 64 + lane;
-  if (st == 1) {
-    half_t* urow = p.u2 ? p.u2 + row * DV : nullptr;
+  const float lam = (float)p.lambda_scale[0];
 #pragma unroll
-    for (int tt = 0; tt < NOT; ++tt)
+  for (int qs = 0; qs < QS; ++qs) {
+    const float lsum = pair_sum(l[qs]);
+    const float inv = 1.0f / lsum;
+    const size_t row = (size_t)bh * p.N + qrow0 + 32 * qs;
+    {
+      float* lse = st ? p.lse2 : p.lse1;
+      if (g == 0 && lse) lse[row] = (m[qs] + __builtin_log2f(lsum)) * kLn2;
+    }
+    // stream-2 waves hand softmax(S2)V to the stream-1 wave that owns the same rows (same lane,
+    // same register index), through the now idle tile memory
+    float* xchg = reinterpret_cast<float*>(smem) + (size_t)(qw * QS + qs) * NOT * 16 * 64 + lane;
+    if (st == 1) {
+      half_t* urow = p.u2 ? p.u2 + row * DV : nullptr;
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        h4 uv;
+      for (int tt = 0; tt < NOT; ++tt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float u = o[tt][4 * r4 + e] * inv;
-          xchg[(tt * 16 + 4 * r4 + e) * 64] = u;
-          uv[e] = (half_t)u;
+        for (int r4 = 0; r4 < 4; ++r4) {
+          h4 uv;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            float u = o[qs][tt][4 * r4 + e] * inv;
+            xchg[(tt * 16 + 4 * r4 + e) * 64] = u;
+            uv[e] = (half_t)u;
+          }
+          if (urow) *reinterpret_cast<h4*>(urow + 32 * tt + 8 * r4 + 4 * g) = uv;
         }
-        if (urow) *reinterpret_cast<h4*>(urow + 32 * tt + 8 * r4 + 4 * g) = uv;
-      }
+    } else {
+#pragma unroll
+      for (int tt = 0; tt < NOT; ++tt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[qs][tt][r] *= inv;
+    }
   }
   __syncthreads();
   if (st == 0) {
-    const float lam = (float)p.lambda_scale[0];
-    float ss = 0.f;
 #pragma unroll
-    for (int tt = 0; tt < NOT; ++tt)
+    for (int qs = 0; qs < QS; ++qs) {
+      const size_t row = (size_t)bh * p.N + qrow0 + 32 * qs;
+      const float* xchg = reinterpret_cast<const float*>(smem) + (size_t)(qw * QS + qs) * NOT * 16 * 64 + lane;
+      float ss = 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float x = o[tt][r] * inv - lam * xchg[(tt * 16 + r) * 64];
-        o[tt][r] = x;
-        ss += x * x;
+      for (int tt = 0; tt < NOT; ++tt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float x = o[qs][tt][r] - lam * xchg[(tt * 16 + r) * 64];
+          o[qs][tt][r] = x;
+          ss += x * x;
+        }
+      float scale = 1.0f;
+      if (RMS) {
+        ss = pair_sum(ss);
+        const float rr = __builtin_amdgcn_rsqf(ss * (1.0f / DV) + kEps);
+        scale = (1.0f - p.lambda_init) * rr;
+        if (g == 0 && p.rinv) p.rinv[row] = rr;
       }
-    float scale = 1.0f;
-    if (RMS) {
-      ss = pair_sum(ss);
-      const float rr = __builtin_amdgcn_rsqf(ss * (1.0f / DV) + kEps);
-      scale = (1.0f - p.lambda_init) * rr;
-      if (g == 0 && p.rinv) p.rinv[row] = rr;
+      half_t* yrow = p.y + row * DV;
+#pragma unroll
+      for (int tt = 0; tt < NOT; ++tt)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          h4 yv;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) yv[e] = (half_t)(o[qs][tt][4 * r4 + e] * scale);
+          *reinterpret_cast<h4*>(yrow + 32 * tt + 8 * r4 + 4 * g) = yv;
+        }
     }
-    half_t* yrow = p.y + row * DV;
-#pragma unroll
-    for (int tt = 0; tt < NOT; ++tt)
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        h4 yv;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) yv[e] = (half_t)(o[tt][4 * r4 + e] * scale);
-        *reinterpret_cast<h4*>(yrow + 32 * tt + 8 * r4 + 4 * g) = yv;
-      }
   }
 }
 
