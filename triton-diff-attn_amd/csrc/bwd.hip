@@ -113,21 +113,23 @@ __global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restric
 template <int D>
 struct DkvCfg {
   static constexpr int DV = 2 * D;
-  static constexpr int NT = 256;
-  static constexpr int BK = 128;               // keys per workgroup (32 per wave)
-  static constexpr int BQ = 64;                // query rows per staged tile
-  static constexpr int QS = D + 8;             // LDS row strides (halfs)
-  static constexpr int XS = DV + 8;
-  static constexpr int Q_TILE = BQ * QS;
-  static constexpr int X_TILE = BQ * XS;
+  static constexpr int NW = 4;                 // waves per workgroup, 32 keys each
+  static constexpr int NT = NW * 64;
+  static constexpr int BK = NW * 32;           // keys per workgroup
+  static constexpr int BQ = (D <= 64) ? 64 : 32;  // query rows per staged tile
+  static constexpr int Q_TILE = BQ * D;        // halfs (swizzled, unpadded)
+  static constexpr int X_TILE = BQ * DV;
   static constexpr int STAT = 4 * BQ * 2;      // 4 float arrays, counted in halfs
   static constexpr int STAGE = 2 * Q_TILE + X_TILE + STAT;
 };
 
+// dK_t and dV for one block of keys.  Products are formed as [queries x keys] so that a lane owns
+// one key column; P and dS in accumulator layout are then directly the A operands (rows = keys,
+// contraction over queries) of dV = P^T dX and dK_t = dS_t^T Q_t.
 template <int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_kernel(BwdParams p) {
+__global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_kernel(BwdParams p) {
   using C = DkvCfg<D>;
-  constexpr int DV = C::DV, NT = C::NT, BK = C::BK, BQ = C::BQ, QS = C::QS, XS = C::XS;
+  constexpr int DV = C::DV, NW = C::NW, BK = C::BK, BQ = C::BQ;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32, NVT = DV / 32;
 
   __shared__ __attribute__((aligned(16))) half_t smem[2 * C::STAGE];
@@ -171,38 +173,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dk1[t][r] = 0.f; dk2[t][r] = 0.f; }
 
-  TileStage<BQ, D, QS, NT> stQ1, stQ2;
-  TileStage<BQ, DV, XS, NT> stX;
-  float st_stat = 0.f;
+  using QTile = AsyncTile<BQ, D, NW>;
+  using XTile = AsyncTile<BQ, DV, NW>;
   const half_t* gq1 = p.q1 + row0 * D;
   const half_t* gq2 = p.q2 + row0 * D;
   const half_t* gx = p.dx + row0 * DV;
-  // thread t stages stat[t / BQ][t % BQ]  (4 * BQ = 256 = NT values)
-  const float* gstat = p.stat + (size_t)(tid / BQ) * rows + row0 + (tid % BQ);
+  // the 4 x BQ statistics of a query tile are one piece of 16*BQ bytes: lane l < BQ fetches
+  // stat[l / (BQ/4)][4 * (l % (BQ/4)) .. +3]
+  const float* gstat = p.stat + (size_t)(lane / (BQ / 4)) * rows + row0 + 4 * (lane % (BQ / 4));
+  constexpr int XH = (XTile::PER + 1) / 2;
 
-  auto stage_load = [&](int qt) {
-    stQ1.load(gq1 + (size_t)qt * BQ * D, tid);
-    stQ2.load(gq2 + (size_t)qt * BQ * D, tid);
-    stX.load(gx + (size_t)qt * BQ * DV, tid);
-    st_stat = gstat[(size_t)qt * BQ];
-  };
-  auto stage_store = [&](int buf) {
+  auto stage = [&](int qt, int buf, int part) {
     half_t* b = smem + buf * C::STAGE;
-    stQ1.store(b, tid);
-    stQ2.store(b + C::Q_TILE, tid);
-    stX.store(b + 2 * C::Q_TILE, tid);
-    reinterpret_cast<float*>(b + 2 * C::Q_TILE + C::X_TILE)[tid] = st_stat;
+    if (part == 0) {
+      QTile::issue(gq1 + (size_t)qt * BQ * D, b, wave, lane);
+      if (wave == 0 && lane < BQ) async_copy16(reinterpret_cast<const half_t*>(gstat + (size_t)qt * BQ), b + 2 * C::Q_TILE + C::X_TILE);
+    } else if (part == 1) {
+      QTile::issue(gq2 + (size_t)qt * BQ * D, b + C::Q_TILE, wave, lane);
+    } else if (part == 2) {
+      XTile::template issue<0, XH>(gx + (size_t)qt * BQ * DV, b + 2 * C::Q_TILE, wave, lane);
+    } else {
+      XTile::template issue<XH, XTile::PER>(gx + (size_t)qt * BQ * DV, b + 2 * C::Q_TILE, wave, lane);
+    }
   };
 
-  stage_load(0);
-  stage_store(0);
-  __syncthreads();
-
-  // per-lane LDS offsets (halfs)
-  const int a_q = j * QS + 8 * g;                 // A fragment of Q (row = query j)
-  const int a_x = j * XS + 8 * g;                 // A fragment of dX
   const int tr_row = 4 * g + ((lane & 15) >> 2);  // transposing reads: row inside a 16-row k-step
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  stage(0, 0, 0); stage(0, 0, 1); stage(0, 0, 2); stage(0, 0, 3);
+  wait_async_tiles();
+  __syncthreads();
 
   const int n_qt = p.N / BQ;
   for (int qt = 0; qt < n_qt; ++qt) {
@@ -210,7 +210,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const half_t* sQ2 = sQ1 + C::Q_TILE;
     const half_t* sX = sQ1 + 2 * C::Q_TILE;
     const float* sStat = reinterpret_cast<const float*>(sQ1 + 2 * C::Q_TILE + C::X_TILE);
-    stage_load((qt + 1 < n_qt) ? qt + 1 : qt);   // the last iteration re-reads its own tile: harmless
+    const int qn = (qt + 1 < n_qt) ? qt + 1 : qt;   // the last iteration re-reads its own tile: harmless
+    const int nbuf = (qt + 1) & 1;
+    stage(qn, nbuf, 0);
 
 #pragma unroll
     for (int qs = 0; qs < BQ / 32; ++qs) {
@@ -219,16 +221,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       for (int r = 0; r < 16; ++r) { s1[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
-        h8 a1 = *reinterpret_cast<const h8*>(sQ1 + qs * 32 * QS + a_q + 16 * ks);
+        h8 a1 = *reinterpret_cast<const h8*>(sQ1 + swz_off<D>(qs * 32 + j, 16 * ks + 8 * g));
         s1 = mfma32(a1, kf1[ks], s1);
-        h8 a2 = *reinterpret_cast<const h8*>(sQ2 + qs * 32 * QS + a_q + 16 * ks);
+        h8 a2 = *reinterpret_cast<const h8*>(sQ2 + swz_off<D>(qs * 32 + j, 16 * ks + 8 * g));
         s2 = mfma32(a2, kf2[ks], s2);
       }
 #pragma unroll
       for (int kv = 0; kv < NKV; ++kv) {
-        h8 a = *reinterpret_cast<const h8*>(sX + qs * 32 * XS + a_x + 16 * kv);
+        h8 a = *reinterpret_cast<const h8*>(sX + swz_off<DV>(qs * 32 + j, 16 * kv + 8 * g));
         dp = mfma32(a, vf[kv], dp);
       }
+      if (qs == 0) { stage(qn, nbuf, 1); stage(qn, nbuf, 2); }
+      if (qs == BQ / 32 - 1) stage(qn, nbuf, 3);
       // registers r of the 32x32 tiles hold query rows 8*(r/4) + 4g + (r%4)
       h8 pc[2], d1[2], d2[2];
 #pragma unroll
@@ -244,8 +248,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           const float p1 = fast_exp2(__builtin_fmaf(s1[r], c, nl1[e]));
           const float p2 = fast_exp2(__builtin_fmaf(s2[r], c, nl2[e]));
           const float ds1 = p1 * (dp[r] - de1[e]);
-          const float ds2 = p2 * (-lam * dp[r] - de2[e]);
-          pc[r / 8][r % 8] = (half_t)(p1 - lam * p2);
+          const float ds2 = p2 * __builtin_fmaf(-lam, dp[r], -de2[e]);
+          pc[r / 8][r % 8] = (half_t)__builtin_fmaf(-lam, p2, p1);
           d1[r / 8][r % 8] = (half_t)ds1;
           d2[r / 8][r % 8] = (half_t)ds2;
         }
@@ -255,23 +259,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         const int rbase = qs * 32 + 16 * kk + tr_row;
 #pragma unroll
         for (int tt = 0; tt < NVT; ++tt) {
-          const half_t* bp = sX + rbase * XS + 32 * tt + tr_col;
-          h8 b = join(lds_read_tr(bp), lds_read_tr(bp + 8 * XS));
+          h8 b = join(lds_read_tr(sX + swz_off<DV>(rbase, 32 * tt + tr_col)),
+                      lds_read_tr(sX + swz_off<DV>(rbase + 8, 32 * tt + tr_col)));
           dv[tt] = mfma32(pc[kk], b, dv[tt]);
         }
 #pragma unroll
         for (int tt = 0; tt < NDT; ++tt) {
-          const half_t* b1p = sQ1 + rbase * QS + 32 * tt + tr_col;
-          h8 b1 = join(lds_read_tr(b1p), lds_read_tr(b1p + 8 * QS));
+          h8 b1 = join(lds_read_tr(sQ1 + swz_off<D>(rbase, 32 * tt + tr_col)),
+                       lds_read_tr(sQ1 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
           dk1[tt] = mfma32(d1[kk], b1, dk1[tt]);
-          const half_t* b2p = sQ2 + rbase * QS + 32 * tt + tr_col;
-          h8 b2 = join(lds_read_tr(b2p), lds_read_tr(b2p + 8 * QS));
+          h8 b2 = join(lds_read_tr(sQ2 + swz_off<D>(rbase, 32 * tt + tr_col)),
+                       lds_read_tr(sQ2 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
           dk2[tt] = mfma32(d2[kk], b2, dk2[tt]);
         }
       }
     }
 
-    stage_store((qt + 1) & 1);
+    wait_async_tiles();
     __syncthreads();
   }
 
@@ -298,20 +302,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 template <int D>
 struct DqCfg {
   static constexpr int DV = 2 * D;
-  static constexpr int NT = 256;
-  static constexpr int BM = 128;               // query rows per workgroup (32 per wave)
+  static constexpr int NW = 4;                 // waves per workgroup, 32 query rows each
+  static constexpr int NT = NW * 64;
+  static constexpr int BM = NW * 32;           // query rows per workgroup
   static constexpr int BN = (D <= 64) ? 64 : 32;  // keys per staged tile
-  static constexpr int KS = D + 8;
-  static constexpr int VS = DV + 8;
-  static constexpr int K_TILE = BN * KS;
-  static constexpr int V_TILE = BN * VS;
+  static constexpr int K_TILE = BN * D;        // halfs (swizzled, unpadded)
+  static constexpr int V_TILE = BN * DV;
   static constexpr int STAGE = 2 * K_TILE + V_TILE;
 };
 
+// dQ_t = s * dS_t K_t for one block of query rows.  Every product is formed transposed,
+// [keys x queries], so that a lane owns one query column: the row statistics are per-lane
+// scalars and dS^T in accumulator layout is directly the B operand of dQ^T = K^T dS^T.
 template <int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(DqCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<D>;
-  constexpr int DV = C::DV, NT = C::NT, BM = C::BM, BN = C::BN, KS = C::KS, VS = C::VS;
+  constexpr int DV = C::DV, NW = C::NW, BM = C::BM, BN = C::BN;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
 
   __shared__ __attribute__((aligned(16))) half_t smem[2 * C::STAGE];
@@ -327,19 +333,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const size_t row0 = (size_t)bh * p.N;
   const size_t qrow = row0 + qt * BM + wave * 32 + j;
 
-  const float c = p.sm_scale * kLog2e;
   const float lam = (float)p.lambda_scale[0];
 
-  // persistent B operands: this lane's query row of Q1, Q2, dX, and its row statistics
+  // persistent B operands: this lane's query row of Q1, Q2 (pre-multiplied by sm_scale*log2(e)
+  // exactly as in the forward kernel, so the recomputed probabilities match it), dX, and its row
+  // statistics
   h8 qf1[NKS], qf2[NKS], xf[NKV];
   {
+    const float c = p.sm_scale * kLog2e;
     const half_t* r1 = p.q1 + qrow * D + 8 * g;
     const half_t* r2 = p.q2 + qrow * D + 8 * g;
     const half_t* rx = p.dx + qrow * DV + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
-      qf1[ks] = *reinterpret_cast<const h8*>(r1 + 16 * ks);
-      qf2[ks] = *reinterpret_cast<const h8*>(r2 + 16 * ks);
+      h8 a = *reinterpret_cast<const h8*>(r1 + 16 * ks);
+      h8 b = *reinterpret_cast<const h8*>(r2 + 16 * ks);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { a[e] = (half_t)((float)a[e] * c); b[e] = (half_t)((float)b[e] * c); }
+      qf1[ks] = a; qf2[ks] = b;
     }
 #pragma unroll
     for (int kv = 0; kv < NKV; ++kv) xf[kv] = *reinterpret_cast<const h8*>(rx + 16 * kv);
@@ -353,80 +364,82 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dq1[t][r] = 0.f; dq2[t][r] = 0.f; }
 
-  TileStage<BN, D, KS, NT> stK1, stK2;
-  TileStage<BN, DV, VS, NT> stV;
+  using KTile = AsyncTile<BN, D, NW>;
+  using VTile = AsyncTile<BN, DV, NW>;
   const half_t* gk1 = p.k1 + row0 * D;
   const half_t* gk2 = p.k2 + row0 * D;
   const half_t* gv = p.v + row0 * DV;
+  const int n_tiles = p.N / BN;
+  constexpr int VH = (VTile::PER + 1) / 2;
 
-  stK1.load(gk1, tid); stK2.load(gk2, tid); stV.load(gv, tid);
-  stK1.store(smem, tid); stK2.store(smem + C::K_TILE, tid); stV.store(smem + 2 * C::K_TILE, tid);
+  KTile::issue(gk1, smem, wave, lane);
+  KTile::issue(gk2, smem + C::K_TILE, wave, lane);
+  VTile::issue(gv, smem + 2 * C::K_TILE, wave, lane);
+  wait_async_tiles();
   __syncthreads();
 
-  const int a_k = j * KS + 8 * g;                 // A fragment of K (row = key j)
-  const int a_v = j * VS + 8 * g;                 // A fragment of V
   const int tr_row = 4 * g + ((lane & 15) >> 2);
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  const int n_tiles = p.N / BN;
   for (int t = 0; t < n_tiles; ++t) {
     const half_t* sK1 = smem + (t & 1) * C::STAGE;
     const half_t* sK2 = sK1 + C::K_TILE;
     const half_t* sV = sK1 + 2 * C::K_TILE;
+    half_t* nb = smem + ((t + 1) & 1) * C::STAGE;
     const int tn = (t + 1 < n_tiles) ? t + 1 : t;   // the last iteration re-reads its own tile: harmless
-    stK1.load(gk1 + (size_t)tn * BN * D, tid);
-    stK2.load(gk2 + (size_t)tn * BN * D, tid);
-    stV.load(gv + (size_t)tn * BN * DV, tid);
+    KTile::issue(gk1 + (size_t)tn * BN * D, nb, wave, lane);
 
 #pragma unroll
     for (int ksub = 0; ksub < BN / 32; ++ksub) {
+      if (ksub == 0) KTile::issue(gk2 + (size_t)tn * BN * D, nb + C::K_TILE, wave, lane);
       // transposed tiles [32 keys x 32 queries]: this lane's column is its query
       f16v s1, s2, dp;
 #pragma unroll
       for (int r = 0; r < 16; ++r) { s1[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
-        h8 a1 = *reinterpret_cast<const h8*>(sK1 + ksub * 32 * KS + a_k + 16 * ks);
+        h8 a1 = *reinterpret_cast<const h8*>(sK1 + swz_off<D>(ksub * 32 + j, 16 * ks + 8 * g));
         s1 = mfma32(a1, qf1[ks], s1);
-        h8 a2 = *reinterpret_cast<const h8*>(sK2 + ksub * 32 * KS + a_k + 16 * ks);
+        h8 a2 = *reinterpret_cast<const h8*>(sK2 + swz_off<D>(ksub * 32 + j, 16 * ks + 8 * g));
         s2 = mfma32(a2, qf2[ks], s2);
       }
 #pragma unroll
       for (int kv = 0; kv < NKV; ++kv) {
-        h8 a = *reinterpret_cast<const h8*>(sV + ksub * 32 * VS + a_v + 16 * kv);
+        h8 a = *reinterpret_cast<const h8*>(sV + swz_off<DV>(ksub * 32 + j, 16 * kv + 8 * g));
         dp = mfma32(a, xf[kv], dp);
       }
+      if (ksub == 0) VTile::template issue<0, VH>(gv + (size_t)tn * BN * DV, nb + 2 * C::K_TILE, wave, lane);
+      if (ksub == BN / 32 - 1) VTile::template issue<VH, VTile::PER>(gv + (size_t)tn * BN * DV, nb + 2 * C::K_TILE, wave, lane);
       h8 b1[2], b2[2];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float p1 = fast_exp2(__builtin_fmaf(s1[r], c, nl1));
-        const float p2 = fast_exp2(__builtin_fmaf(s2[r], c, nl2));
+        const float p1 = fast_exp2(s1[r] + nl1);
+        const float p2 = fast_exp2(s2[r] + nl2);
         b1[r / 8][r % 8] = (half_t)(p1 * (dp[r] - de1));
-        b2[r / 8][r % 8] = (half_t)(p2 * (-lam * dp[r] - de2));
+        b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dp[r], -de2));
       }
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
         const int rbase = ksub * 32 + 16 * kk + tr_row;
 #pragma unroll
         for (int tt = 0; tt < NDT; ++tt) {
-          const half_t* a1p = sK1 + rbase * KS + 32 * tt + tr_col;
-          h8 a1 = join(lds_read_tr(a1p), lds_read_tr(a1p + 8 * KS));
+          h8 a1 = join(lds_read_tr(sK1 + swz_off<D>(rbase, 32 * tt + tr_col)),
+                       lds_read_tr(sK1 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
           dq1[tt] = mfma32(a1, b1[kk], dq1[tt]);
-          const half_t* a2p = sK2 + rbase * KS + 32 * tt + tr_col;
-          h8 a2 = join(lds_read_tr(a2p), lds_read_tr(a2p + 8 * KS));
+          h8 a2 = join(lds_read_tr(sK2 + swz_off<D>(rbase, 32 * tt + tr_col)),
+                       lds_read_tr(sK2 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
           dq2[tt] = mfma32(a2, b2[kk], dq2[tt]);
         }
       }
     }
 
-    {
-      half_t* nb = smem + ((t + 1) & 1) * C::STAGE;
-      stK1.store(nb, tid); stK2.store(nb + C::K_TILE, tid); stV.store(nb + 2 * C::K_TILE, tid);
-    }
+    wait_async_tiles();
     __syncthreads();
   }
 
-  // dQ^T tile tt: this lane's column is its query; register r = feature 32*tt + 8*(r/4) + 4g + (r%4)
+  // dQ^T tile tt: this lane's column is its query; register r = feature 32*tt + 8*(r/4) + 4g + (r%4).
+  // The accumulated sums carry log2(e) from the pre-scaled Q only inside the probabilities, so the
+  // remaining factor is the plain softmax scale.
   half_t* o1 = p.dq1 + qrow * D;
   half_t* o2 = p.dq2 + qrow * D;
 #pragma unroll
@@ -461,11 +474,11 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 4u) {
-    hipLaunchKernelGGL((bwd_dkdv_kernel<D>), dim3(p.BH * (p.N / DkvCfg<D>::BK)), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((bwd_dkdv_kernel<D>), dim3(p.BH * (p.N / DkvCfg<D>::BK)), dim3(DkvCfg<D>::NT), 0, stream, p);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 8u) {
-    hipLaunchKernelGGL((bwd_dq_kernel<D>), dim3(p.BH * (p.N / DqCfg<D>::BM)), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((bwd_dq_kernel<D>), dim3(p.BH * (p.N / DqCfg<D>::BM)), dim3(DqCfg<D>::NT), 0, stream, p);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   return e;
