@@ -29,7 +29,7 @@ struct FwdCfg {
   static constexpr int V_TILE = BN * DV;
   static constexpr int K_BUF = 2 * K_TILE;         // K1 and K2 of one tile
   static constexpr int TILES = 2 * K_BUF + 2 * V_TILE;       // two K buffers and two V buffers
-  static constexpr int XCHG = (BM / 32) * (DV / 32) * 16 * 64 * 2;   // halfs needed by the epilogue exchange
+  static constexpr int XCHG = NW * 32 * (DV + 8);            // halfs needed by the epilogue staging blocks
   static constexpr int SMEM = (TILES > XCHG) ? TILES : XCHG;
 };
 
@@ -252,75 +252,77 @@ void fwd_kernel(FwdParams p) {
     iteration(t + 1, s_b, s_a);
   }
 
-  // ---- epilogue: every quantity below is per query = per lane pair (l, l^32) ----
-  const float lam = (float)p.lambda_scale[0];
+  // ---- epilogue ----------------------------------------------------------------------------
+  // Every row quantity is per query = per lane pair (l, l^32).  Each wave owns a staging block of
+  // 32 rows x DV halfs in the now idle tile memory (row stride DV+8 halfs).  Results are written
+  // there in accumulator layout (8 bytes per lane) and read back row by row, so that the global
+  // stores are whole 16-byte chunks of consecutive rows.  The stream-2 waves stage softmax(S2)V
+  // rounded to fp16 -- the tensor saved for backward -- and the stream-1 wave that owns the same
+  // rows reads it from there for the lambda-combine.
+  constexpr int SROW = DV + 8;
+  half_t* const stg_own = smem + (size_t)wave * 32 * SROW;
+  auto stage_rows = [&](int qs, const f16v (&val)[NOT], float scale) {
 #pragma unroll
-  for (int qs = 0; qs < QS; ++qs) {
-    const float lsum = pair_sum(l[qs]);
-    const float inv = 1.0f / lsum;
-    const size_t row = (size_t)bh * p.N + qrow0 + 32 * qs;
-    {
-      float* lse = st ? p.lse2 : p.lse1;
-      if (g == 0 && lse) lse[row] = (m[qs] + __builtin_log2f(lsum)) * kLn2;
+    for (int tt = 0; tt < NOT; ++tt)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        h4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (half_t)(val[tt][4 * r4 + e] * scale);
+        *reinterpret_cast<h4*>(stg_own + j * SROW + 32 * tt + 8 * r4 + 4 * g) = v;
+      }
+    (void)qs;
+  };
+  auto store_rows = [&](half_t* gbase /* first of this wave's 32 rows */) {
+    constexpr int LPR = DV / 8;            // lanes per row
+    constexpr int RPI = 64 / LPR;          // rows per instruction
+#pragma unroll
+    for (int k = 0; k < 32 / RPI; ++k) {
+      const int row = k * RPI + lane / LPR, ch = lane % LPR;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stg_own + row * SROW + 8 * ch);
+      *reinterpret_cast<u32x4*>(gbase + (size_t)row * DV + 8 * ch) = v;
     }
-    // stream-2 waves hand softmax(S2)V to the stream-1 wave that owns the same rows (same lane,
-    // same register index), through the now idle tile memory
-    float* xchg = reinterpret_cast<float*>(smem) + (size_t)(qw * QS + qs) * NOT * 16 * 64 + lane;
-    if (st == 1) {
-      half_t* urow = p.u2 ? p.u2 + row * DV : nullptr;
-#pragma unroll
-      for (int tt = 0; tt < NOT; ++tt)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          h4 uv;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            float u = o[qs][tt][4 * r4 + e] * inv;
-            xchg[(tt * 16 + 4 * r4 + e) * 64] = u;
-            uv[e] = (half_t)u;
-          }
-          if (urow) *reinterpret_cast<h4*>(urow + 32 * tt + 8 * r4 + 4 * g) = uv;
-        }
-    } else {
-#pragma unroll
-      for (int tt = 0; tt < NOT; ++tt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[qs][tt][r] *= inv;
-    }
+  };
+
+  static_assert(QS == 1, "the epilogue stages one 32-row block per wave");
+  const float lsum = pair_sum(l[0]);
+  const float inv = 1.0f / lsum;
+  const size_t row = (size_t)bh * p.N + qrow0;
+  const size_t wave_row0 = (size_t)bh * p.N + qt * BM + qw * 32;
+  {
+    float* lse = st ? p.lse2 : p.lse1;
+    if (g == 0 && lse) lse[row] = (m[0] + __builtin_log2f(lsum)) * kLn2;
   }
+  if (st == 1) stage_rows(0, o[0], inv);
   __syncthreads();
-  if (st == 0) {
+  if (st == 1) {
+    if (p.u2) store_rows(p.u2 + wave_row0 * DV);
+  } else {
+    const float lam = (float)p.lambda_scale[0];
+    const half_t* stg_u2 = smem + (size_t)(wave + NW / 2) * 32 * SROW;
+    float ss = 0.f;
 #pragma unroll
-    for (int qs = 0; qs < QS; ++qs) {
-      const size_t row = (size_t)bh * p.N + qrow0 + 32 * qs;
-      const float* xchg = reinterpret_cast<const float*>(smem) + (size_t)(qw * QS + qs) * NOT * 16 * 64 + lane;
-      float ss = 0.f;
+    for (int tt = 0; tt < NOT; ++tt)
 #pragma unroll
-      for (int tt = 0; tt < NOT; ++tt)
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const h4 u = *reinterpret_cast<const h4*>(stg_u2 + j * SROW + 32 * tt + 8 * r4 + 4 * g);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float x = o[qs][tt][r] - lam * xchg[(tt * 16 + r) * 64];
-          o[qs][tt][r] = x;
+        for (int e = 0; e < 4; ++e) {
+          const float x = o[0][tt][4 * r4 + e] * inv - lam * (float)u[e];
+          o[0][tt][4 * r4 + e] = x;
           ss += x * x;
         }
-      float scale = 1.0f;
-      if (RMS) {
-        ss = pair_sum(ss);
-        const float rr = __builtin_amdgcn_rsqf(ss * (1.0f / DV) + kEps);
-        scale = (1.0f - p.lambda_init) * rr;
-        if (g == 0 && p.rinv) p.rinv[row] = rr;
       }
-      half_t* yrow = p.y + row * DV;
-#pragma unroll
-      for (int tt = 0; tt < NOT; ++tt)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          h4 yv;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) yv[e] = (half_t)(o[qs][tt][4 * r4 + e] * scale);
-          *reinterpret_cast<h4*>(yrow + 32 * tt + 8 * r4 + 4 * g) = yv;
-        }
+    float scale = 1.0f;
+    if (RMS) {
+      ss = pair_sum(ss);
+      const float rr = __builtin_amdgcn_rsqf(ss * (1.0f / DV) + kEps);
+      scale = (1.0f - p.lambda_init) * rr;
+      if (g == 0 && p.rinv) p.rinv[row] = rr;
     }
+    stage_rows(0, o[0], scale);
+    __builtin_amdgcn_wave_barrier();   // the rows are read back by other lanes of this wave only
+    store_rows(p.y + wave_row0 * DV);
   }
 }
 
