@@ -84,8 +84,8 @@ def cpu_baseline(cfg, torch, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
@@ -164,9 +164,15 @@ def main():
     unit = B * H * N * N * D
     dkdv_flops = 16 * unit      # S1,S2 (4) + dP (4) + dV (4) + dK1,dK2 (4), times B*H*N^2*D
     dkdv_tflops = dkdv_flops / (kernels_ms["bwd_dkdv_kernel"] * 1e-3) / 1e12
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic_headline_B4H32N2048D64.json")
+    if args.workload == "headline" and os.path.exists(tpath):
+        # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the file's note)
+        k = json.load(open(tpath))["kernels"]["bwd_dkdv_kernel"]
+        traffic = k["fetch_bytes"] + k["write_bytes"]
     roofline = {
         "bound": "mfma", "kernel": "bwd_dkdv_kernel", "achieved": dkdv_tflops, "peak": PEAK_FP16_TFLOPS,
-        "unit": "TFLOP/s", "frac": dkdv_tflops / PEAK_FP16_TFLOPS, "traffic": None,
+        "unit": "TFLOP/s", "frac": dkdv_tflops / PEAK_FP16_TFLOPS, "traffic": traffic,
         "flops_per_launch": dkdv_flops, "ms_per_launch": kernels_ms["bwd_dkdv_kernel"],
     }
 
