@@ -115,6 +115,13 @@ struct AsyncTile {
     const int row = L / CPR, cpos = L % CPR;
     return row * COLS + ((cpos ^ swz_f<CPR>(row)) << 3);
   }
+  // number of instructions wave `wave` issues for one tile
+  __device__ static __forceinline__ int count(int wave) {
+    int n = 0;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) n += (wave + NW * k < NINST) ? 1 : 0;
+    return n;
+  }
   // issues this wave's instructions k0 .. k1-1 (of PER) for the tile
   template <int K0 = 0, int K1 = PER>
   __device__ static __forceinline__ void issue(const half_t* gtile, half_t* lds_tile, int wave, int lane) {
@@ -128,6 +135,22 @@ struct AsyncTile {
 };
 
 __device__ __forceinline__ void wait_async_tiles() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Waits until at most `newest` (wave-uniform, 0..8) of this wave's vector-memory loads are still in
+// flight.  Loads complete in issue order, so this is "everything except the last `newest` issued".
+__device__ __forceinline__ void wait_async_tiles_except(int newest) {
+  switch (newest) {
+    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+    case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+  }
+}
 
 // Cooperative copy of a dense [ROWS x COLS] fp16 tile (row stride COLS in global memory) into an
 // LDS tile with row stride STRIDE, staged through registers so the global loads of the next tile

@@ -28,7 +28,8 @@ struct FwdCfg {
   static constexpr int K_TILE = BN * D;            // halfs, one stream (swizzled, unpadded)
   static constexpr int V_TILE = BN * DV;
   static constexpr int K_BUF = 2 * K_TILE;         // K1 and K2 of one tile
-  static constexpr int TILES = 2 * K_BUF + 2 * V_TILE;       // two K buffers and two V buffers
+  static constexpr int NBUF = 3;                   // ring depth: tiles are fetched two iterations ahead
+  static constexpr int TILES = NBUF * (K_BUF + V_TILE);
   static constexpr int XCHG = NW * 32 * (DV + 8);            // halfs needed by the epilogue staging blocks
   static constexpr int SMEM = (TILES > XCHG) ? TILES : XCHG;
 };
@@ -46,8 +47,8 @@ void fwd_kernel(FwdParams p) {
   constexpr int NOT = DV / 32;               // 32-row tiles of O^T
 
   __shared__ __attribute__((aligned(16))) half_t smem[C::SMEM];
-  half_t* const sKbuf = smem;                       // [2][K1 tile, K2 tile]
-  half_t* const sVbuf = smem + 2 * C::K_BUF;        // [2][V tile]
+  half_t* const sKbuf = smem;                              // [NBUF][K1 tile, K2 tile]
+  half_t* const sVbuf = smem + C::NBUF * C::K_BUF;         // [NBUF][V tile]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -128,10 +129,14 @@ void fwd_kernel(FwdParams p) {
       }
   };
 
-  // prologue: K tiles 0 and 1 and V tile 0; scores of tile 0
-  load_k1(0, 0); load_k2(0, 0);
-  load_k1((n_tiles > 1) ? 1 : 0, 1); load_k2((n_tiles > 1) ? 1 : 0, 1);
-  load_va(0, 0); load_vb(0, 0);
+  // loads this wave issues per iteration (one K1, one K2 and one V tile)
+  const int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
+  auto clampt = [&](int t) { return t < n_tiles ? t : n_tiles - 1; };   // past the end: harmless re-reads
+
+  // prologue: K tiles 0..2 and V tiles 0..1; scores of tile 0
+  load_k1(0, 0); load_k2(0, 0); load_va(0, 0); load_vb(0, 0);
+  load_k1(clampt(1), 1); load_k2(clampt(1), 1); load_va(clampt(1), 1); load_vb(clampt(1), 1);
+  load_k1(clampt(2), 2); load_k2(clampt(2), 2);
   wait_async_tiles();
   __syncthreads();
   f16v s_a[QS][NKT], s_b[QS][NKT];
@@ -141,6 +146,10 @@ void fwd_kernel(FwdParams p) {
     scores(ka, s_a);
   }
   __syncthreads();   // K buffer 0 is overwritten by the first iteration's prefetch
+  // ring positions: K tile t+1 is read from kb1, V tile t from vb0; K tile t+3 goes to kb0 (tile t,
+  // consumed one iteration ago), V tile t+2 to vb2 (tile t-1, likewise)
+  int kb0 = 0, kb1 = 1, vb0 = 0, vb2 = 2;
+  auto advance = [](int& b) { b = (b == 2) ? 0 : b + 1; };
 
   // transposing-read coordinates of this lane inside a 16-key k-step: key row and feature column
   const int tr_row = 4 * g + ((lane & 15) >> 2);
@@ -149,18 +158,17 @@ void fwd_kernel(FwdParams p) {
   // One iteration: softmax of tile t (scores in s_cur) and its P*V product, overlapped with the score
   // product of tile t+1 (into s_nxt).
   auto iteration = [&](int t, f16v (&s_cur)[QS][NKT], f16v (&s_nxt)[QS][NKT]) {
-    // Asynchronous prefetch straight into LDS: K tile t+2 replaces K tile t (consumed one iteration
-    // ago), V tile t+1 replaces V tile t-1 (clamped at the end: harmless re-reads).  The groups of
-    // load instructions are spread over the iteration so that the waves do not queue up behind each
-    // other at the memory pipeline.
-    const int tk = (t + 2 < n_tiles) ? t + 2 : n_tiles - 1;
-    const int tv = (t + 1 < n_tiles) ? t + 1 : n_tiles - 1;
-    load_k1(tk, t & 1);
+    // Asynchronous prefetch straight into LDS, two iterations ahead: K tile t+3 and V tile t+2.
+    // The groups of load instructions are spread over the iteration so that the waves do not
+    // queue up behind each other at the memory pipeline.
+    const int tk = clampt(t + 3);
+    const int tv = clampt(t + 2);
+    load_k1(tk, kb0);
 
     // K fragments of the next tile are requested first; the row maxima of this tile are reduced
     // while they arrive.
     h8 ka[NKT][NKS];
-    read_k(sKbuf + ((t + 1) & 1) * C::K_BUF + st * C::K_TILE, ka);
+    read_k(sKbuf + kb1 * C::K_BUF + st * C::K_TILE, ka);
 
     float mx[QS];
 #pragma unroll
@@ -206,7 +214,7 @@ void fwd_kernel(FwdParams p) {
 
     // From here on one basic block: the score product of the next tile and the P*V product of this
     // tile run on the matrix unit while the exponentials run on the VALU.
-    load_k2(tk, t & 1);
+    load_k2(tk, kb0);
     scores(ka, s_nxt);
 
     h8 pb[QS][NKK];      // P^T as B operands: pb[kk] covers keys 16kk..16kk+15 (accumulator order)
@@ -228,11 +236,11 @@ void fwd_kernel(FwdParams p) {
       l[qs] += rs;
     }
 
-    const half_t* sV = sVbuf + (t & 1) * C::V_TILE;
+    const half_t* sV = sVbuf + vb0 * C::V_TILE;
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {
-      if (kk == 0) load_va(tv, (t + 1) & 1);
-      if (kk == NKK / 2) load_vb(tv, (t + 1) & 1);
+      if (kk == 0) load_va(tv, vb2);
+      if (kk == NKK / 2) load_vb(tv, vb2);
 #pragma unroll
       for (int tt = 0; tt < NOT; ++tt) {
         h8 a = join(lds_read_tr(sV + swz_off<DV>(16 * kk + tr_row, 32 * tt + tr_col)),
@@ -242,8 +250,10 @@ void fwd_kernel(FwdParams p) {
       }
     }
 
-    wait_async_tiles();
+    // the tiles needed next were requested one iteration ago: only this iteration's loads may remain
+    wait_async_tiles_except(loads_per_iter);
     __syncthreads();
+    advance(kb0); advance(kb1); advance(vb0); advance(vb2);
   };
 
   // the tile count is even (N is a multiple of 128, tiles are at most 64 keys)
@@ -252,6 +262,8 @@ void fwd_kernel(FwdParams p) {
     iteration(t + 1, s_b, s_a);
   }
 
+  wait_async_tiles();   // the staging blocks below reuse the tile memory the last prefetches write to
+  __syncthreads();
   // ---- epilogue ----------------------------------------------------------------------------
   // Every row quantity is per query = per lane pair (l, l^32).  Each wave owns a staging block of
   // 32 rows x DV halfs in the now idle tile memory (row stride DV+8 halfs).  Results are written
