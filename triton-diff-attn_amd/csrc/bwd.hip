@@ -13,6 +13,8 @@
 //
 // The pre-norm row X is rebuilt as Y / ((1 - lambda_init) * rinv); only U2 = softmax(S2) V is
 // needed besides it, because U1 = X + lambda U2.
+#include <type_traits>
+
 #include "params.hpp"
 
 namespace da {
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   constexpr int DV = C::DV, NW = C::NW, BK = C::BK, BQ = C::BQ;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32, NVT = DV / 32;
 
-  __shared__ __attribute__((aligned(16))) half_t smem[2 * C::STAGE];
+  __shared__ __attribute__((aligned(16))) half_t smem[3 * C::STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -200,83 +202,159 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   const int tr_row = 4 * g + ((lane & 15) >> 2);  // transposing reads: row inside a 16-row k-step
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
+  // The loop runs over 32-query sub-tiles i (SPT per staged tile), software-pipelined inside the
+  // wave.  Step i interleaves, instruction group by instruction group,
+  //   the 16 matrix products S1, S2, dP of sub-tile i+1     (matrix unit, A fragments from LDS)
+  //   the element-wise work of sub-tile i, one register row per product   (VALU)
+  // and then issues the 16 products dV, dK1, dK2 of sub-tile i.  The interleaving is written out in
+  // source order and pinned with scheduling barriers, because the matrix products with
+  // AGPR-resident B fragments are opaque to the instruction scheduler.
+  // A staged tile is read one step after its last sub-tile was scored: three stage buffers.
+  constexpr int SPT = BQ / 32;
+  struct Scores { f16v s1, s2, dp; };
+  struct Packed { h8 pc[2], d1[2], d2[2]; };   // A operands of the dV / dK1 / dK2 products
+  constexpr int NPROD = 2 * NKS + NKV;         // matrix products per sub-tile in the first phase
+  constexpr int DEPTH = 4;                     // A fragments requested ahead of their product
+
+  // A fragment of product k of sub-tile qs in buffer buf: k < 2*NKS alternates Q1/Q2 k-steps, then dX
+  auto prod_frag = [&](int buf, int qs, int k) -> h8 {
+    const half_t* sQ1 = smem + buf * C::STAGE;
+    if (k < 2 * NKS) {
+      const half_t* sQ = sQ1 + (k & 1) * C::Q_TILE;
+      return *reinterpret_cast<const h8*>(sQ + swz_off<D>(qs * 32 + j, 16 * (k >> 1) + 8 * g));
+    }
+    return *reinterpret_cast<const h8*>(sQ1 + 2 * C::Q_TILE + swz_off<DV>(qs * 32 + j, 16 * (k - 2 * NKS) + 8 * g));
+  };
+  auto prod_mfma = [&](int k, h8 a, Scores& out) {
+    if (k < 2 * NKS) {
+      const int ks = k >> 1;
+      if (k & 1) out.s2 = ks ? mfma32_bagpr(a, kf2[ks], out.s2) : mfma32_bagpr_first(a, kf2[ks]);
+      else       out.s1 = ks ? mfma32_bagpr(a, kf1[ks], out.s1) : mfma32_bagpr_first(a, kf1[ks]);
+    } else {
+      const int kv = k - 2 * NKS;
+      out.dp = kv ? mfma32_bagpr(a, vf[kv], out.dp) : mfma32_bagpr_first(a, vf[kv]);
+    }
+  };
+  // row statistics of the four query rows 8*r4 + 4g .. +3 of sub-tile qs: {-lse1', -lse2', delta1, delta2}
+  struct Stat4 { f4v nl1, nl2, de1, de2; };
+  auto load_stats = [&](int buf, int qs, int r4) -> Stat4 {
+    const float* sStat = reinterpret_cast<const float*>(smem + buf * C::STAGE + 2 * C::Q_TILE + C::X_TILE) + qs * 32 + 8 * r4 + 4 * g;
+    Stat4 s;
+    s.nl1 = *reinterpret_cast<const f4v*>(sStat + 0 * BQ);
+    s.nl2 = *reinterpret_cast<const f4v*>(sStat + 1 * BQ);
+    s.de1 = *reinterpret_cast<const f4v*>(sStat + 2 * BQ);
+    s.de2 = *reinterpret_cast<const f4v*>(sStat + 3 * BQ);
+    return s;
+  };
+  // element-wise work of accumulator register r (query row 8*(r/4) + 4g + (r%4))
+  auto elementwise = [&](int r, const Stat4& st, const Scores& in, Packed& out) {
+    const int e = r % 4;
+    const float p1 = fast_exp2(__builtin_fmaf(in.s1[r], c, st.nl1[e]));
+    const float p2 = fast_exp2(__builtin_fmaf(in.s2[r], c, st.nl2[e]));
+    const float ds1 = p1 * (in.dp[r] - st.de1[e]);
+    const float ds2 = p2 * __builtin_fmaf(-lam, in.dp[r], -st.de2[e]);
+    out.pc[r / 8][r % 8] = (half_t)__builtin_fmaf(-lam, p2, p1);
+    out.d1[r / 8][r % 8] = (half_t)ds1;
+    out.d2[r / 8][r % 8] = (half_t)ds2;
+  };
+  // B fragment (transposing read) of accumulate product m of sub-tile qs: m = kk*(NVT+2*NDT) + slot
+  constexpr int NACC1 = NVT + 2 * NDT;         // products per 16-query k-step
+  auto acc_frag = [&](int buf, int qs, int m) -> h8 {
+    const half_t* sQ1 = smem + buf * C::STAGE;
+    const int kk = m / NACC1, slot = m % NACC1;
+    const int rbase = qs * 32 + 16 * kk + tr_row;
+    if (slot < NVT) {
+      const half_t* sX = sQ1 + 2 * C::Q_TILE;
+      return join(lds_read_tr(sX + swz_off<DV>(rbase, 32 * slot + tr_col)),
+                  lds_read_tr(sX + swz_off<DV>(rbase + 8, 32 * slot + tr_col)));
+    }
+    const int t2 = slot - NVT;
+    const half_t* sQ = sQ1 + (t2 & 1) * C::Q_TILE;
+    return join(lds_read_tr(sQ + swz_off<D>(rbase, 32 * (t2 >> 1) + tr_col)),
+                lds_read_tr(sQ + swz_off<D>(rbase + 8, 32 * (t2 >> 1) + tr_col)));
+  };
+  auto acc_mfma = [&](int m, h8 bfrag, const Packed& in) {
+    const int kk = m / NACC1, slot = m % NACC1;
+    if (slot < NVT) { dv[slot] = mfma32(in.pc[kk], bfrag, dv[slot]); return; }
+    const int t2 = slot - NVT;
+    if (t2 & 1) dk2[t2 >> 1] = mfma32(in.d2[kk], bfrag, dk2[t2 >> 1]);
+    else        dk1[t2 >> 1] = mfma32(in.d1[kk], bfrag, dk1[t2 >> 1]);
+  };
+  auto accumulate = [&](int buf, int qs, const Packed& in) {
+    constexpr int NACC = 2 * NACC1, AD = 3;    // B fragments are requested AD products ahead
+    h8 bf[NACC];
+#pragma unroll
+    for (int m = 0; m < AD; ++m) bf[m] = acc_frag(buf, qs, m);
+#pragma unroll
+    for (int m = 0; m < NACC; ++m) {
+      if (m + AD < NACC) bf[m + AD] = acc_frag(buf, qs, m + AD);
+      acc_mfma(m, bf[m], in);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  const int n_qt = p.N / BQ;
+  const int n_sub = p.N / 32;
+  auto buf_of = [](int tile) { return tile % 3; };
+
+  // products of sub-tile (bufn, qsn) interleaved with the element-wise work of sub-tile (bufc, qsc):
+  // one accumulator register row per product; fragments and statistics are requested ahead
+  static_assert(NPROD % 16 == 0 || 16 % NPROD == 0, "rows are spread evenly over the products");
+  auto fused = [&](int bufn, int qsn, Scores& s_nxt, int bufc, int qsc, const Scores& s_cur, Packed& p_cur) {
+    h8 a[NPROD];
+    Stat4 st[4];
+#pragma unroll
+    for (int k = 0; k < DEPTH; ++k) a[k] = prod_frag(bufn, qsn, k);
+    st[0] = load_stats(bufc, qsc, 0);
+#pragma unroll
+    for (int k = 0; k < NPROD; ++k) {
+      if (k + DEPTH < NPROD) a[k + DEPTH] = prod_frag(bufn, qsn, k + DEPTH);
+      const int r0 = 16 * k / NPROD, r1 = 16 * (k + 1) / NPROD;
+      // statistics of the next group of four rows, one group ahead
+      if (r0 % 4 == 0 && r1 > r0 && r0 / 4 + 1 < 4) st[r0 / 4 + 1] = load_stats(bufc, qsc, r0 / 4 + 1);
+      prod_mfma(k, a[k], s_nxt);
+#pragma unroll
+      for (int r = r0; r < r1; ++r) elementwise(r, st[r / 4], s_cur, p_cur);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  // step i: compile-time position SUBN of sub-tile i+1 inside its tile
+  auto step = [&](int i, auto subn_tag, const Scores& s_cur, Scores& s_nxt, Packed& p_cur) {
+    constexpr int SUBN = decltype(subn_tag)::value;           // (i + 1) % SPT
+    constexpr int SUBC = (SUBN + SPT - 1) % SPT;              // i % SPT
+    const bool more = (i + 1 < n_sub);
+    const int tn = (more ? i + 1 : i) / SPT, tc = i / SPT;
+    if (SUBN == 0 && more) {
+      // sub-tile i+1 opens tile tn: its data must have landed; then fetch tile tn+1
+      wait_async_tiles();
+      __syncthreads();
+      const int tl = (tn + 1 < n_qt) ? tn + 1 : tn;           // past the end: harmless re-read
+      stage(tl, buf_of(tn + 1), 0); stage(tl, buf_of(tn + 1), 1);
+      stage(tl, buf_of(tn + 1), 2); stage(tl, buf_of(tn + 1), 3);
+    }
+    // past the end the last sub-tile is scored again and the result is never used
+    fused(buf_of(tn), more ? SUBN : SUBC, s_nxt, buf_of(tc), SUBC, s_cur, p_cur);
+    accumulate(buf_of(tc), SUBC, p_cur);
+  };
+
+  // prologue: tile 0, then start fetching tile 1; scores of sub-tile 0
   stage(0, 0, 0); stage(0, 0, 1); stage(0, 0, 2); stage(0, 0, 3);
   wait_async_tiles();
   __syncthreads();
+  {
+    const int t1 = (n_qt > 1) ? 1 : 0;
+    stage(t1, 1, 0); stage(t1, 1, 1); stage(t1, 1, 2); stage(t1, 1, 3);
+  }
+  Scores sa, sb;
+  Packed pk;
+#pragma unroll
+  for (int k = 0; k < NPROD; ++k) prod_mfma(k, prod_frag(0, 0, k), sa);
+  mfma_results_ready(sa.s1, sa.s2, sa.dp);
 
-  const int n_qt = p.N / BQ;
-  for (int qt = 0; qt < n_qt; ++qt) {
-    const half_t* sQ1 = smem + (qt & 1) * C::STAGE;
-    const half_t* sQ2 = sQ1 + C::Q_TILE;
-    const half_t* sX = sQ1 + 2 * C::Q_TILE;
-    const float* sStat = reinterpret_cast<const float*>(sQ1 + 2 * C::Q_TILE + C::X_TILE);
-    const int qn = (qt + 1 < n_qt) ? qt + 1 : qt;   // the last iteration re-reads its own tile: harmless
-    const int nbuf = (qt + 1) & 1;
-    stage(qn, nbuf, 0);
-
-#pragma unroll
-    for (int qs = 0; qs < BQ / 32; ++qs) {
-      f16v s1, s2, dp;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { s1[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
-#pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        h8 a1 = *reinterpret_cast<const h8*>(sQ1 + swz_off<D>(qs * 32 + j, 16 * ks + 8 * g));
-        s1 = mfma32(a1, kf1[ks], s1);
-        h8 a2 = *reinterpret_cast<const h8*>(sQ2 + swz_off<D>(qs * 32 + j, 16 * ks + 8 * g));
-        s2 = mfma32(a2, kf2[ks], s2);
-      }
-#pragma unroll
-      for (int kv = 0; kv < NKV; ++kv) {
-        h8 a = *reinterpret_cast<const h8*>(sX + swz_off<DV>(qs * 32 + j, 16 * kv + 8 * g));
-        dp = mfma32(a, vf[kv], dp);
-      }
-      if (qs == 0) { stage(qn, nbuf, 1); stage(qn, nbuf, 2); }
-      if (qs == BQ / 32 - 1) stage(qn, nbuf, 3);
-      // registers r of the 32x32 tiles hold query rows 8*(r/4) + 4g + (r%4)
-      h8 pc[2], d1[2], d2[2];
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const int qo = qs * 32 + 8 * r4 + 4 * g;
-        const f4v nl1 = *reinterpret_cast<const f4v*>(sStat + 0 * BQ + qo);
-        const f4v nl2 = *reinterpret_cast<const f4v*>(sStat + 1 * BQ + qo);
-        const f4v de1 = *reinterpret_cast<const f4v*>(sStat + 2 * BQ + qo);
-        const f4v de2 = *reinterpret_cast<const f4v*>(sStat + 3 * BQ + qo);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 4 * r4 + e;
-          const float p1 = fast_exp2(__builtin_fmaf(s1[r], c, nl1[e]));
-          const float p2 = fast_exp2(__builtin_fmaf(s2[r], c, nl2[e]));
-          const float ds1 = p1 * (dp[r] - de1[e]);
-          const float ds2 = p2 * __builtin_fmaf(-lam, dp[r], -de2[e]);
-          pc[r / 8][r % 8] = (half_t)__builtin_fmaf(-lam, p2, p1);
-          d1[r / 8][r % 8] = (half_t)ds1;
-          d2[r / 8][r % 8] = (half_t)ds2;
-        }
-      }
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const int rbase = qs * 32 + 16 * kk + tr_row;
-#pragma unroll
-        for (int tt = 0; tt < NVT; ++tt) {
-          h8 b = join(lds_read_tr(sX + swz_off<DV>(rbase, 32 * tt + tr_col)),
-                      lds_read_tr(sX + swz_off<DV>(rbase + 8, 32 * tt + tr_col)));
-          dv[tt] = mfma32(pc[kk], b, dv[tt]);
-        }
-#pragma unroll
-        for (int tt = 0; tt < NDT; ++tt) {
-          h8 b1 = join(lds_read_tr(sQ1 + swz_off<D>(rbase, 32 * tt + tr_col)),
-                       lds_read_tr(sQ1 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
-          dk1[tt] = mfma32(d1[kk], b1, dk1[tt]);
-          h8 b2 = join(lds_read_tr(sQ2 + swz_off<D>(rbase, 32 * tt + tr_col)),
-                       lds_read_tr(sQ2 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
-          dk2[tt] = mfma32(d2[kk], b2, dk2[tt]);
-        }
-      }
-    }
-
-    wait_async_tiles();
-    __syncthreads();
+  for (int i = 0; i < n_sub; i += 2) {   // the sub-tile count is even
+    step(i, std::integral_constant<int, 1 % SPT>{}, sa, sb, pk);
+    step(i + 1, std::integral_constant<int, 2 % SPT>{}, sb, sa, pk);
   }
 
   // accumulator tile tt: column = 32*tt + j (feature), register r = key row 8*(r/4) + 4g + (r%4)
@@ -302,13 +380,14 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
 template <int D>
 struct DqCfg {
   static constexpr int DV = 2 * D;
-  static constexpr int NW = 4;                 // waves per workgroup, 32 query rows each
+  static constexpr int NW = 8;                 // waves per workgroup, 32 query rows each
   static constexpr int NT = NW * 64;
   static constexpr int BM = NW * 32;           // query rows per workgroup
   static constexpr int BN = (D <= 64) ? 64 : 32;  // keys per staged tile
   static constexpr int K_TILE = BN * D;        // halfs (swizzled, unpadded)
   static constexpr int V_TILE = BN * DV;
   static constexpr int STAGE = 2 * K_TILE + V_TILE;
+  static constexpr int NBUF = 3;               // ring depth: tiles are fetched two iterations ahead
 };
 
 // dQ_t = s * dS_t K_t for one block of query rows.  Every product is formed transposed,
@@ -320,7 +399,7 @@ __global__ __launch_bounds__(DqCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(2,
   constexpr int DV = C::DV, NW = C::NW, BM = C::BM, BN = C::BN;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
 
-  __shared__ __attribute__((aligned(16))) half_t smem[2 * C::STAGE];
+  __shared__ __attribute__((aligned(16))) half_t smem[C::NBUF * C::STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -372,21 +451,28 @@ __global__ __launch_bounds__(DqCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(2,
   const int n_tiles = p.N / BN;
   constexpr int VH = (VTile::PER + 1) / 2;
 
-  KTile::issue(gk1, smem, wave, lane);
-  KTile::issue(gk2, smem + C::K_TILE, wave, lane);
-  VTile::issue(gv, smem + 2 * C::K_TILE, wave, lane);
-  wait_async_tiles();
+  const int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
+  auto fetch_all = [&](int t, int buf) {
+    half_t* b = smem + buf * C::STAGE;
+    KTile::issue(gk1 + (size_t)t * BN * D, b, wave, lane);
+    KTile::issue(gk2 + (size_t)t * BN * D, b + C::K_TILE, wave, lane);
+    VTile::issue(gv + (size_t)t * BN * DV, b + 2 * C::K_TILE, wave, lane);
+  };
+  fetch_all(0, 0);
+  fetch_all((n_tiles > 1) ? 1 : 0, 1);
+  wait_async_tiles_except(loads_per_iter);   // tile 0 has landed, tile 1 may still be in flight
   __syncthreads();
+  int bcur = 0, bnext = 2;   // buffer of tile t, buffer that receives tile t+2
 
   const int tr_row = 4 * g + ((lane & 15) >> 2);
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   for (int t = 0; t < n_tiles; ++t) {
-    const half_t* sK1 = smem + (t & 1) * C::STAGE;
+    const half_t* sK1 = smem + bcur * C::STAGE;
     const half_t* sK2 = sK1 + C::K_TILE;
     const half_t* sV = sK1 + 2 * C::K_TILE;
-    half_t* nb = smem + ((t + 1) & 1) * C::STAGE;
-    const int tn = (t + 1 < n_tiles) ? t + 1 : t;   // the last iteration re-reads its own tile: harmless
+    half_t* nb = smem + bnext * C::STAGE;            // held tile t-1, consumed one iteration ago
+    const int tn = (t + 2 < n_tiles) ? t + 2 : n_tiles - 1;   // past the end: harmless re-reads
     KTile::issue(gk1 + (size_t)tn * BN * D, nb, wave, lane);
 
 #pragma unroll
@@ -433,9 +519,13 @@ __global__ __launch_bounds__(DqCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(2,
       }
     }
 
-    wait_async_tiles();
+    // tile t+1 was requested one iteration ago: only this iteration's loads may remain in flight
+    wait_async_tiles_except(loads_per_iter);
     __syncthreads();
+    bcur = (bcur == 2) ? 0 : bcur + 1;
+    bnext = (bnext == 2) ? 0 : bnext + 1;
   }
+  wait_async_tiles();
 
   // dQ^T tile tt: this lane's column is its query; register r = feature 32*tt + 8*(r/4) + 4g + (r%4).
   // The accumulated sums carry log2(e) from the pre-scaled Q only inside the probabilities, so the

@@ -33,6 +33,25 @@ __device__ __forceinline__ f16v mfma32(h8 a, h8 b, f16v c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 }
 
+// MFMA with the B operand held in an accumulation register (AGPR) and the result in ordinary
+// VGPRs.  Used where B is a loop-invariant fragment: it then lives in the AGPR half of the register
+// file for the whole kernel, at no cost in VGPRs and without copies.  Being inline assembly, the
+// compiler does not know these are matrix instructions: the caller must put mfma_results_ready()
+// between the last of them and the first VALU read of the result.
+__device__ __forceinline__ f16v mfma32_bagpr_first(h8 a, h8 b) {
+  f16v d;
+  asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+  return d;
+}
+__device__ __forceinline__ f16v mfma32_bagpr(h8 a, h8 b, f16v c) {
+  asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  return c;
+}
+// Wait states that cover the write-back of an 8-pass MFMA before a VALU instruction reads it.
+__device__ __forceinline__ void mfma_results_ready(f16v& x, f16v& y, f16v& z) {
+  asm volatile("s_nop 15\n\ts_nop 3" : "+v"(x), "+v"(y), "+v"(z));
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // v_permlane32_swap exchanges the upper half of its first register with the lower half of its
