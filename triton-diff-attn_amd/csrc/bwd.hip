@@ -377,10 +377,10 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
 }
 
 // ------------------------------------------------------------------------------------------------
-template <int D>
+template <int D, int NWAVES>
 struct DqCfg {
   static constexpr int DV = 2 * D;
-  static constexpr int NW = 8;                 // waves per workgroup, 32 query rows each
+  static constexpr int NW = NWAVES;            // waves per workgroup, 32 query rows each
   static constexpr int NT = NW * 64;
   static constexpr int BM = NW * 32;           // query rows per workgroup
   static constexpr int BN = (D <= 64) ? 64 : 32;  // keys per staged tile
@@ -393,9 +393,9 @@ struct DqCfg {
 // dQ_t = s * dS_t K_t for one block of query rows.  Every product is formed transposed,
 // [keys x queries], so that a lane owns one query column: the row statistics are per-lane
 // scalars and dS^T in accumulator layout is directly the B operand of dQ^T = K^T dS^T.
-template <int D>
-__global__ __launch_bounds__(DqCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_kernel(BwdParams p) {
-  using C = DqCfg<D>;
+template <int D, int NWAVES>
+__global__ __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_kernel(BwdParams p) {
+  using C = DqCfg<D, NWAVES>;
   constexpr int DV = C::DV, NW = C::NW, BM = C::BM, BN = C::BN;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
 
@@ -568,7 +568,11 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 8u) {
-    hipLaunchKernelGGL((bwd_dq_kernel<D>), dim3(p.BH * (p.N / DqCfg<D>::BM)), dim3(DqCfg<D>::NT), 0, stream, p);
+    // 256 query rows per workgroup when the sequence allows it, otherwise 128
+    if (p.N % 256 == 0)
+      hipLaunchKernelGGL((bwd_dq_kernel<D, 8>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
+    else
+      hipLaunchKernelGGL((bwd_dq_kernel<D, 4>), dim3(p.BH * (p.N / 128)), dim3(256), 0, stream, p);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   return e;
