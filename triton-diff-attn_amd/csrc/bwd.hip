@@ -81,8 +81,9 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
       const float delta2 = -lam * t2;
       p.stat[0 * rows + row] = -p.lse1[row] * kLog2e;
       p.stat[1 * rows + row] = -p.lse2[row] * kLog2e;
-      p.stat[2 * rows + row] = tx - delta2;
-      p.stat[3 * rows + row] = delta2;
+      const float delta1 = tx - delta2;
+      p.stat[2 * rows + row] = -delta1;
+      p.stat[3 * rows + row] = -(lam * delta1 + delta2);
       part -= t2;
     }
   }
@@ -123,6 +124,9 @@ struct DkvCfg {
   static constexpr int X_TILE = BQ * DV;
   static constexpr int STAT = 4 * BQ * 2;      // 4 float arrays, counted in halfs
   static constexpr int STAGE = 2 * Q_TILE + X_TILE + STAT;
+  // a staged tile is read until half a step after its last sub-tile was scored while the tile two
+  // ahead is already being fetched: three buffers, four when a tile is a single sub-tile
+  static constexpr int NBUF = (BQ == 32) ? 4 : 3;
 };
 
 // dK_t and dV for one block of keys.  Products are formed as [queries x keys] so that a lane owns
@@ -134,7 +138,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   constexpr int DV = C::DV, NW = C::NW, BK = C::BK, BQ = C::BQ;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32, NVT = DV / 32;
 
-  __shared__ __attribute__((aligned(16))) half_t smem[3 * C::STAGE];
+  __shared__ __attribute__((aligned(16))) half_t smem[C::NBUF * C::STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -158,8 +162,12 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     const half_t* rv = p.v + (row0 + key) * DV + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
-      kf1[ks] = *reinterpret_cast<const h8*>(r1 + 16 * ks);
-      kf2[ks] = *reinterpret_cast<const h8*>(r2 + 16 * ks);
+      // pre-multiplied by sm_scale*log2(e): the score products come out in log2 units
+      h8 x1 = *reinterpret_cast<const h8*>(r1 + 16 * ks);
+      h8 x2 = *reinterpret_cast<const h8*>(r2 + 16 * ks);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { x1[e] = (half_t)((float)x1[e] * c); x2[e] = (half_t)((float)x2[e] * c); }
+      kf1[ks] = x1; kf2[ks] = x2;
     }
 #pragma unroll
     for (int kv = 0; kv < NKV; ++kv) vf[kv] = *reinterpret_cast<const h8*>(rv + 16 * kv);
@@ -204,61 +212,88 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
 
   // The loop runs over 32-query sub-tiles i (SPT per staged tile), software-pipelined inside the
   // wave.  Step i interleaves, instruction group by instruction group,
-  //   the 16 matrix products S1, S2, dP of sub-tile i+1     (matrix unit, A fragments from LDS)
-  //   the element-wise work of sub-tile i, one register row per product   (VALU)
-  // and then issues the 16 products dV, dK1, dK2 of sub-tile i.  The interleaving is written out in
-  // source order and pinned with scheduling barriers, because the matrix products with
-  // AGPR-resident B fragments are opaque to the instruction scheduler.
-  // A staged tile is read one step after its last sub-tile was scored: three stage buffers.
+  //   the matrix products S1, S2, dP of sub-tile i+1          (matrix unit, A fragments from LDS)
+  //   the element-wise work of sub-tile i, one register row at a time          (VALU)
+  //   the products dV, dK1, dK2 over queries 16..31 of sub-tile i-1 during the first half of the
+  //   step and over queries 0..15 of sub-tile i during the second half, as soon as the
+  //   element-wise work has packed their operands              (matrix unit, B fragments from LDS)
+  // The interleaving is written out in source order and pinned with scheduling barriers, because
+  // the matrix products with AGPR-resident B fragments are opaque to the instruction scheduler.
   constexpr int SPT = BQ / 32;
   struct Scores { f16v s1, s2, dp; };
   struct Packed { h8 pc[2], d1[2], d2[2]; };   // A operands of the dV / dK1 / dK2 products
   constexpr int NPROD = 2 * NKS + NKV;         // matrix products per sub-tile in the first phase
-  constexpr int DEPTH = 4;                     // A fragments requested ahead of their product
+  constexpr int DEPTH = 3;                     // A fragments requested ahead of their product
 
-  // A fragment of product k of sub-tile qs in buffer buf: k < 2*NKS alternates Q1/Q2 k-steps, then dX
+  // Product k of a sub-tile: even k is k-step k/2 of dP; odd k alternates k-steps of S1 and S2.
+  // Two products of one chain are never neighbours: a product whose accumulator input is the
+  // result of the product issued just before the previous one was observed to read stale values
+  // when the one in between writes AGPRs.
+  static_assert(NKV == 2 * NKS, "every second product belongs to dP");
   auto prod_frag = [&](int buf, int qs, int k) -> h8 {
     const half_t* sQ1 = smem + buf * C::STAGE;
-    if (k < 2 * NKS) {
-      const half_t* sQ = sQ1 + (k & 1) * C::Q_TILE;
-      return *reinterpret_cast<const h8*>(sQ + swz_off<D>(qs * 32 + j, 16 * (k >> 1) + 8 * g));
+    if (k & 1) {
+      const int t = k >> 1;
+      const half_t* sQ = sQ1 + (t & 1) * C::Q_TILE;
+      return *reinterpret_cast<const h8*>(sQ + swz_off<D>(qs * 32 + j, 16 * (t >> 1) + 8 * g));
     }
-    return *reinterpret_cast<const h8*>(sQ1 + 2 * C::Q_TILE + swz_off<DV>(qs * 32 + j, 16 * (k - 2 * NKS) + 8 * g));
+    return *reinterpret_cast<const h8*>(sQ1 + 2 * C::Q_TILE + swz_off<DV>(qs * 32 + j, 16 * (k >> 1) + 8 * g));
   };
   auto prod_mfma = [&](int k, h8 a, Scores& out) {
-    if (k < 2 * NKS) {
-      const int ks = k >> 1;
-      if (k & 1) out.s2 = ks ? mfma32_bagpr(a, kf2[ks], out.s2) : mfma32_bagpr_first(a, kf2[ks]);
-      else       out.s1 = ks ? mfma32_bagpr(a, kf1[ks], out.s1) : mfma32_bagpr_first(a, kf1[ks]);
+    if (k & 1) {
+      const int t = k >> 1, ks = t >> 1;
+      if (t & 1) out.s2 = mfma32_bagpr(a, kf2[ks], out.s2);
+      else       out.s1 = mfma32_bagpr(a, kf1[ks], out.s1);
     } else {
-      const int kv = k - 2 * NKS;
-      out.dp = kv ? mfma32_bagpr(a, vf[kv], out.dp) : mfma32_bagpr_first(a, vf[kv]);
+      out.dp = mfma32_bagpr(a, vf[k >> 1], out.dp);
     }
   };
-  // row statistics of the four query rows 8*r4 + 4g .. +3 of sub-tile qs: {-lse1', -lse2', delta1, delta2}
-  struct Stat4 { f4v nl1, nl2, de1, de2; };
-  auto load_stats = [&](int buf, int qs, int r4) -> Stat4 {
-    const float* sStat = reinterpret_cast<const float*>(smem + buf * C::STAGE + 2 * C::Q_TILE + C::X_TILE) + qs * 32 + 8 * r4 + 4 * g;
-    Stat4 s;
-    s.nl1 = *reinterpret_cast<const f4v*>(sStat + 0 * BQ);
-    s.nl2 = *reinterpret_cast<const f4v*>(sStat + 1 * BQ);
-    s.de1 = *reinterpret_cast<const f4v*>(sStat + 2 * BQ);
-    s.de2 = *reinterpret_cast<const f4v*>(sStat + 3 * BQ);
-    return s;
+  // Row statistics written by the preprocess kernel: 0: -lse1*log2e, 1: -lse2*log2e, 2: -delta1,
+  // 3: -(lambda*delta1 + delta2).  Statistics 0..2 are the initial accumulator values of the three
+  // product chains, so the matrix unit delivers s1 - lse1, s2 - lse2 (log2 units) and dP - delta1.
+  auto stat4 = [&](int buf, int qs, int which, int r4) -> f4v {
+    const float* sStat = reinterpret_cast<const float*>(smem + buf * C::STAGE + 2 * C::Q_TILE + C::X_TILE);
+    return *reinterpret_cast<const f4v*>(sStat + which * BQ + qs * 32 + 8 * r4 + 4 * g);
   };
-  // element-wise work of accumulator register r (query row 8*(r/4) + 4g + (r%4))
-  auto elementwise = [&](int r, const Stat4& st, const Scores& in, Packed& out) {
-    const int e = r % 4;
-    const float p1 = fast_exp2(__builtin_fmaf(in.s1[r], c, st.nl1[e]));
-    const float p2 = fast_exp2(__builtin_fmaf(in.s2[r], c, st.nl2[e]));
-    const float ds1 = p1 * (in.dp[r] - st.de1[e]);
-    const float ds2 = p2 * __builtin_fmaf(-lam, in.dp[r], -st.de2[e]);
-    out.pc[r / 8][r % 8] = (half_t)__builtin_fmaf(-lam, p2, p1);
-    out.d1[r / 8][r % 8] = (half_t)ds1;
-    out.d2[r / 8][r % 8] = (half_t)ds2;
+  auto init_scores = [&](int buf, int qs, Scores& out) {
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      const f4v a = stat4(buf, qs, 0, r4), bq = stat4(buf, qs, 1, r4), cq = stat4(buf, qs, 2, r4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { out.s1[4 * r4 + e] = a[e]; out.s2[4 * r4 + e] = bq[e]; out.dp[4 * r4 + e] = cq[e]; }
+    }
+  };
+  // Element-wise work of accumulator register r (query row 8*(r/4) + 4g + (r%4)), split in three
+  // stages that are issued one product apart, so that no VALU instruction waits on the one
+  // before it: (1) exponentials, (2) products, (3) fp16 packing of a pair of rows.
+  struct RowTmp { float p1[16], p2[16], u[16], ds1[16], ds2[16], pc[16]; };
+  auto ew1 = [&](int r, const f4v& st3, const Scores& in, RowTmp& t) {
+    t.p1[r] = fast_exp2(in.s1[r]);
+    t.p2[r] = fast_exp2(in.s2[r]);
+    t.u[r] = __builtin_fmaf(-lam, in.dp[r], st3[r % 4]);
+    asm volatile("" : "+v"(t.p1[r]), "+v"(t.p2[r]), "+v"(t.u[r]));   // computed here, not moved to its use
+  };
+  auto ew2 = [&](int r, const Scores& in, RowTmp& t) {
+    t.ds1[r] = t.p1[r] * in.dp[r];
+    t.ds2[r] = t.p2[r] * t.u[r];
+    t.pc[r] = __builtin_fmaf(-lam, t.p2[r], t.p1[r]);
+    asm volatile("" : "+v"(t.ds1[r]), "+v"(t.ds2[r]), "+v"(t.pc[r]));
+  };
+  auto ew3 = [&](int r, const RowTmp& t, Packed& out) {   // r odd: packs rows r-1 and r
+    out.pc[r / 8][r % 8 - 1] = (half_t)t.pc[r - 1]; out.pc[r / 8][r % 8] = (half_t)t.pc[r];
+    out.d1[r / 8][r % 8 - 1] = (half_t)t.ds1[r - 1]; out.d1[r / 8][r % 8] = (half_t)t.ds1[r];
+    out.d2[r / 8][r % 8 - 1] = (half_t)t.ds2[r - 1]; out.d2[r / 8][r % 8] = (half_t)t.ds2[r];
+  };
+  // slot s of the skewed schedule: stage 1 of row s, stage 2 of row s-1, stage 3 of the pair ending at row s-2
+  auto ew_slot = [&](int s, const f4v (&st)[4], const Scores& in, RowTmp& t, Packed& out) {
+    if (s < 16) ew1(s, st[s / 4], in, t);
+    if (s >= 1 && s - 1 < 16) ew2(s - 1, in, t);
+    if (s >= 2 && s - 2 < 16 && ((s - 2) & 1)) ew3(s - 2, t, out);
   };
   // B fragment (transposing read) of accumulate product m of sub-tile qs: m = kk*(NVT+2*NDT) + slot
   constexpr int NACC1 = NVT + 2 * NDT;         // products per 16-query k-step
+  constexpr int NACC = 2 * NACC1;
+  static_assert(NACC == NPROD, "one accumulate product per score product");
   auto acc_frag = [&](int buf, int qs, int m) -> h8 {
     const half_t* sQ1 = smem + buf * C::STAGE;
     const int kk = m / NACC1, slot = m % NACC1;
@@ -280,62 +315,80 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     if (t2 & 1) dk2[t2 >> 1] = mfma32(in.d2[kk], bfrag, dk2[t2 >> 1]);
     else        dk1[t2 >> 1] = mfma32(in.d1[kk], bfrag, dk1[t2 >> 1]);
   };
-  auto accumulate = [&](int buf, int qs, const Packed& in) {
-    constexpr int NACC = 2 * NACC1, AD = 3;    // B fragments are requested AD products ahead
-    h8 bf[NACC];
-#pragma unroll
-    for (int m = 0; m < AD; ++m) bf[m] = acc_frag(buf, qs, m);
-#pragma unroll
-    for (int m = 0; m < NACC; ++m) {
-      if (m + AD < NACC) bf[m + AD] = acc_frag(buf, qs, m + AD);
-      acc_mfma(m, bf[m], in);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
 
   const int n_qt = p.N / BQ;
   const int n_sub = p.N / 32;
-  auto buf_of = [](int tile) { return tile % 3; };
+  auto buf_of = [](int tile) { return tile % C::NBUF; };
 
-  // products of sub-tile (bufn, qsn) interleaved with the element-wise work of sub-tile (bufc, qsc):
-  // one accumulator register row per product; fragments and statistics are requested ahead
+  // One step.  Chunk k holds score product k of sub-tile (bufn, qsn), accumulate product
+  // (k + NACC/2) % NACC -- the upper query half of sub-tile (bufp, qsp) while k < NACC/2, then the
+  // lower query half of sub-tile (bufc, qsc) -- and its share of the element-wise rows of sub-tile
+  // (bufc, qsc).  `pk` holds the packed operands: its lower half is written during the first half
+  // of the step and read during the second, its upper half is written during the second half and
+  // read during the first half of the next step.
   static_assert(NPROD % 16 == 0 || 16 % NPROD == 0, "rows are spread evenly over the products");
-  auto fused = [&](int bufn, int qsn, Scores& s_nxt, int bufc, int qsc, const Scores& s_cur, Packed& p_cur) {
-    h8 a[NPROD];
-    Stat4 st[4];
+  constexpr int AHEAD = 3;                     // B fragments requested ahead of their product
+  auto fused = [&](int bufn, int qsn, Scores& s_nxt, int bufc, int qsc, const Scores& s_cur, Packed& pk,
+                   int bufp, int qsp, int tile_next, int buf_next, bool fetch) {
+    constexpr int NSLOT = 18;                  // 16 rows + 2 slots of pipeline drain
+    constexpr int LEAD = 2;                    // slots run before the first product
+    // rows 0..7 are packed by slot 9, which must precede the first product that reads them
+    static_assert(LEAD + (NSLOT - LEAD) * (NPROD / 2) / NPROD > 9, "lower half packed before it is read");
+    auto bfrag = [&](int k) -> h8 {
+      const int m = (k + NACC / 2) % NACC;
+      return (k < NACC / 2) ? acc_frag(bufp, qsp, m) : acc_frag(bufc, qsc, m);
+    };
+    h8 a[NPROD], bf[NACC];
+    f4v st[4];
+    RowTmp tmp;
+    init_scores(bufn, qsn, s_nxt);
 #pragma unroll
     for (int k = 0; k < DEPTH; ++k) a[k] = prod_frag(bufn, qsn, k);
-    st[0] = load_stats(bufc, qsc, 0);
+    st[0] = stat4(bufc, qsc, 3, 0);
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) bf[k] = bfrag(k);
+    // the first slots run while the initial accumulator values and the first fragments arrive
+#pragma unroll
+    for (int s = 0; s < LEAD; ++s) ew_slot(s, st, s_cur, tmp, pk);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int k = 0; k < NPROD; ++k) {
       if (k + DEPTH < NPROD) a[k + DEPTH] = prod_frag(bufn, qsn, k + DEPTH);
-      const int r0 = 16 * k / NPROD, r1 = 16 * (k + 1) / NPROD;
-      // statistics of the next group of four rows, one group ahead
-      if (r0 % 4 == 0 && r1 > r0 && r0 / 4 + 1 < 4) st[r0 / 4 + 1] = load_stats(bufc, qsc, r0 / 4 + 1);
+      if (k + AHEAD < NACC) bf[k + AHEAD] = bfrag(k + AHEAD);
+      // statistics of the next row group, requested a quarter of a step ahead of their use
+      if (k % (NPROD / 4) == 0 && k / (NPROD / 4) < 3) st[k / (NPROD / 4) + 1] = stat4(bufc, qsc, 3, k / (NPROD / 4) + 1);
+      // the next tile's fetch is spread over the products so that the waves do not queue up at the memory pipeline
+      if (fetch && k % (NPROD / 4) == 1) stage(tile_next, buf_next, k / (NPROD / 4));
       prod_mfma(k, a[k], s_nxt);
+      acc_mfma((k + NACC / 2) % NACC, bf[k], pk);
+      // slots LEAD .. NSLOT-1 spread over the products
+      const int s0 = LEAD + (NSLOT - LEAD) * k / NPROD, s1 = LEAD + (NSLOT - LEAD) * (k + 1) / NPROD;
 #pragma unroll
-      for (int r = r0; r < r1; ++r) elementwise(r, st[r / 4], s_cur, p_cur);
+      for (int s = s0; s < s1; ++s) ew_slot(s, st, s_cur, tmp, pk);
       __builtin_amdgcn_sched_barrier(0);
     }
+    // the next step's VALU reads these results right away
+    mfma_results_ready(s_nxt.s1, s_nxt.s2, s_nxt.dp);
   };
 
-  // step i: compile-time position SUBN of sub-tile i+1 inside its tile
-  auto step = [&](int i, auto subn_tag, const Scores& s_cur, Scores& s_nxt, Packed& p_cur) {
+  // step i: compile-time positions of sub-tiles i+1, i, i-1 inside their tiles
+  auto step = [&](int i, auto subn_tag, const Scores& s_cur, Scores& s_nxt, Packed& pk) {
     constexpr int SUBN = decltype(subn_tag)::value;           // (i + 1) % SPT
     constexpr int SUBC = (SUBN + SPT - 1) % SPT;              // i % SPT
+    constexpr int SUBP = (SUBN + 2 * SPT - 2) % SPT;          // (i - 1) % SPT
     const bool more = (i + 1 < n_sub);
-    const int tn = (more ? i + 1 : i) / SPT, tc = i / SPT;
-    if (SUBN == 0 && more) {
-      // sub-tile i+1 opens tile tn: its data must have landed; then fetch tile tn+1
+    const int tn = (more ? i + 1 : i) / SPT, tc = i / SPT, tp = (i > 0 ? i - 1 : 0) / SPT;
+    const bool opens = (SUBN == 0 && more);
+    if (opens) {
+      // sub-tile i+1 opens tile tn: its data must have landed; tile tn+1 is fetched during this step
       wait_async_tiles();
       __syncthreads();
-      const int tl = (tn + 1 < n_qt) ? tn + 1 : tn;           // past the end: harmless re-read
-      stage(tl, buf_of(tn + 1), 0); stage(tl, buf_of(tn + 1), 1);
-      stage(tl, buf_of(tn + 1), 2); stage(tl, buf_of(tn + 1), 3);
     }
-    // past the end the last sub-tile is scored again and the result is never used
-    fused(buf_of(tn), more ? SUBN : SUBC, s_nxt, buf_of(tc), SUBC, s_cur, p_cur);
-    accumulate(buf_of(tc), SUBC, p_cur);
+    const int tl = (tn + 1 < n_qt) ? tn + 1 : tn;             // past the end: harmless re-read
+    // past the end the last sub-tile is scored again and the result is never used; before the
+    // start the all-zero upper operand half is accumulated against tile 0
+    fused(buf_of(tn), more ? SUBN : SUBC, s_nxt, buf_of(tc), SUBC, s_cur, pk,
+          buf_of(tp), (i > 0) ? SUBP : 0, tl, buf_of(tn + 1), opens);
   };
 
   // prologue: tile 0, then start fetching tile 1; scores of sub-tile 0
@@ -349,6 +402,11 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   Scores sa, sb;
   Packed pk;
 #pragma unroll
+  for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { pk.pc[kk][e] = (half_t)0.f; pk.d1[kk][e] = (half_t)0.f; pk.d2[kk][e] = (half_t)0.f; }
+  init_scores(0, 0, sa);
+#pragma unroll
   for (int k = 0; k < NPROD; ++k) prod_mfma(k, prod_frag(0, 0, k), sa);
   mfma_results_ready(sa.s1, sa.s2, sa.dp);
 
@@ -356,6 +414,9 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     step(i, std::integral_constant<int, 1 % SPT>{}, sa, sb, pk);
     step(i + 1, std::integral_constant<int, 2 % SPT>{}, sb, sa, pk);
   }
+  // upper query half of the last sub-tile
+#pragma unroll
+  for (int m = NACC / 2; m < NACC; ++m) acc_mfma(m, acc_frag(buf_of((n_sub - 1) / SPT), (n_sub - 1) % SPT, m), pk);
 
   // accumulator tile tt: column = 32*tt + j (feature), register r = key row 8*(r/4) + 4g + (r%4)
   const size_t krow0 = row0 + (size_t)kt * BK + wave * 32;
@@ -501,8 +562,9 @@ __global__ __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 
       for (int r = 0; r < 16; ++r) {
         const float p1 = fast_exp2(s1[r] + nl1);
         const float p2 = fast_exp2(s2[r] + nl2);
-        b1[r / 8][r % 8] = (half_t)(p1 * (dp[r] - de1));
-        b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dp[r], -de2));
+        const float dpc = dp[r] + de1;                  // statistic 2 is -delta1
+        b1[r / 8][r % 8] = (half_t)(p1 * dpc);
+        b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dpc, de2));   // statistic 3 is -(lambda*delta1 + delta2)
       }
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {

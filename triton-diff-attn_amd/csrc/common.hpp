@@ -44,7 +44,7 @@ __device__ __forceinline__ f16v mfma32_bagpr_first(h8 a, h8 b) {
   return d;
 }
 __device__ __forceinline__ f16v mfma32_bagpr(h8 a, h8 b, f16v c) {
-  asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
   return c;
 }
 // Wait states that cover the write-back of an 8-pass MFMA before a VALU instruction reads it.

@@ -27,7 +27,7 @@ struct BwdParams {
   half_t* dlambda;              // 1 element
   // workspace carve-up
   half_t* dx;                   // [BH,N,2D] gradient w.r.t. the pre-norm rows, fp16
-  float* stat;                  // [4][BH*N]: -lse1*log2(e), -lse2*log2(e), delta1, delta2
+  float* stat;                  // [4][BH*N]: -lse1*log2(e), -lse2*log2(e), -delta1, -(lambda*delta1 + delta2)
   float* dlam_part;             // [n_part] per-workgroup partial sums of d(lambda)
   int n_part;
   int BH, N;
