@@ -190,14 +190,15 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   const half_t* gx = p.dx + row0 * DV;
   // the 4 x BQ statistics of a query tile are one piece of 16*BQ bytes: lane l < BQ fetches
   // stat[l / (BQ/4)][4 * (l % (BQ/4)) .. +3]
-  const float* gstat = p.stat + (size_t)(lane / (BQ / 4)) * rows + row0 + 4 * (lane % (BQ / 4));
+  const float* gstat = p.stat + row0;
+  const unsigned stat_off = (unsigned)(((size_t)(lane / (BQ / 4)) * rows + 4 * (lane % (BQ / 4))) * sizeof(float));
   constexpr int XH = (XTile::PER + 1) / 2;
 
   auto stage = [&](int qt, int buf, int part) {
     half_t* b = smem + buf * C::STAGE;
     if (part == 0) {
       QTile::issue(gq1 + (size_t)qt * BQ * D, b, wave, lane);
-      if (wave == 0 && lane < BQ) async_copy16(reinterpret_cast<const half_t*>(gstat + (size_t)qt * BQ), b + 2 * C::Q_TILE + C::X_TILE);
+      if (wave == 0 && lane < BQ) async_copy16(reinterpret_cast<const half_t*>(gstat + (size_t)qt * BQ), stat_off, b + 2 * C::Q_TILE + C::X_TILE);
     } else if (part == 1) {
       QTile::issue(gq2 + (size_t)qt * BQ * D, b + C::Q_TILE, wave, lane);
     } else if (part == 2) {

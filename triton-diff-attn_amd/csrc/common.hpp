@@ -107,32 +107,38 @@ __device__ __forceinline__ int swz_off(int row, int col) {
   return row * COLS + ((((col >> 3) ^ swz_f<CPR>(row))) << 3) + (col & 7);
 }
 
-// One direct global->LDS load of 16 bytes per lane: lane l's bytes land at lds_base + 16*l, where
-// lds_base must be wave-uniform.  Written as inline assembly so that the compiler's wait-count
-// insertion does not serialise later, unrelated LDS reads behind it; the caller orders it with
-// wait_async_tiles() and a barrier before the data is read.
-__device__ __forceinline__ void async_copy16(const half_t* g, half_t* lds_base) {
+// One direct global->LDS load of 16 bytes per lane: lane l reads g_base + byte_off(l) and its
+// bytes land at lds_base + 16*l; g_base and lds_base must be wave-uniform (they travel in scalar
+// registers, so the per-lane address costs no vector arithmetic).  Written as inline assembly so
+// that the compiler's wait-count insertion does not serialise later, unrelated LDS reads behind
+// it; the caller orders it with wait_async_tiles() and a barrier before the data is read.
+__device__ __forceinline__ void async_copy16(const half_t* g_base, unsigned byte_off, half_t* lds_base) {
   const unsigned lds_addr = (unsigned)(unsigned long)((DA_LDS char*)lds_base);
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-               :: "v"(g), "s"(lds_addr) : "memory");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(byte_off), "s"(g_base), "s"(lds_addr) : "memory");
 }
 
 // Asynchronous copy of a dense [ROWS x COLS] fp16 tile (row stride COLS in global memory) into a
 // swizzled LDS tile with direct global->LDS loads: no registers, no LDS store instructions.  One
-// wave-instruction moves 64 chunks; the hardware writes lane l's 16 bytes at (wave-uniform LDS
-// base) + 16*l, so the swizzle is applied by choosing which global chunk each lane fetches.  NW
-// waves share the tile's instructions round-robin.  Completion: s_waitcnt vmcnt(0), then a barrier.
+// wave-instruction moves 64 chunks (1 KiB, contiguous in global memory as well); the hardware
+// writes lane l's 16 bytes at (wave-uniform LDS base) + 16*l, so the swizzle is applied by
+// choosing which global chunk of the 1 KiB piece each lane fetches.  NW waves share the tile's
+// instructions round-robin.  Completion: s_waitcnt vmcnt(0), then a barrier.
 template <int ROWS, int COLS, int NW>
 struct AsyncTile {
   static constexpr int CPR = COLS / 8;
   static constexpr int NINST = ROWS * CPR / 64;
   static constexpr int PER = (NINST + NW - 1) / NW;
   static_assert((ROWS * CPR) % 64 == 0, "tile must be a whole number of 1 KiB pieces");
-  // global offset (halfs) inside the tile of the chunk that `lane` of `wave` fetches in its k-th instruction
-  __device__ static __forceinline__ int goff(int wave, int lane, int k) {
-    const int L = (wave + NW * k) * 64 + lane;
+  // The swizzle of a piece depends on the piece index only through a few low bits; when the
+  // wave's pieces (wave, wave + NW, ...) agree in those bits, one per-lane offset serves them all.
+  static constexpr bool kOneOffset = (CPR == 4) || (CPR == 8 && NW % 2 == 0) || (CPR == 16 && NW % 4 == 0) ||
+                                     (CPR == 32 && NW % 8 == 0);
+  // byte offset inside piece `inst` of the chunk that `lane` fetches
+  __device__ static __forceinline__ unsigned lane_off(int inst, int lane) {
+    const int L = inst * 64 + lane;
     const int row = L / CPR, cpos = L % CPR;
-    return row * COLS + ((cpos ^ swz_f<CPR>(row)) << 3);
+    return (unsigned)((row * COLS + ((cpos ^ swz_f<CPR>(row)) << 3) - inst * 512) * 2);
   }
   // number of instructions wave `wave` issues for one tile
   __device__ static __forceinline__ int count(int wave) {
@@ -141,15 +147,19 @@ struct AsyncTile {
     for (int k = 0; k < PER; ++k) n += (wave + NW * k < NINST) ? 1 : 0;
     return n;
   }
-  // issues this wave's instructions k0 .. k1-1 (of PER) for the tile
+  // issues this wave's instructions k0 .. k1-1 (of PER) for the tile; `off0` = lane_off(wave, lane)
   template <int K0 = 0, int K1 = PER>
-  __device__ static __forceinline__ void issue(const half_t* gtile, half_t* lds_tile, int wave, int lane) {
+  __device__ static __forceinline__ void issue_at(const half_t* gtile, half_t* lds_tile, int wave, int lane, unsigned off0) {
 #pragma unroll
     for (int k = K0; k < K1; ++k) {
       const int inst = wave + NW * k;
       if (NINST % NW == 0 || inst < NINST)
-        async_copy16(gtile + goff(wave, lane, k), lds_tile + inst * 512);
+        async_copy16(gtile + inst * 512, kOneOffset ? off0 : lane_off(inst, lane), lds_tile + inst * 512);
     }
+  }
+  template <int K0 = 0, int K1 = PER>
+  __device__ static __forceinline__ void issue(const half_t* gtile, half_t* lds_tile, int wave, int lane) {
+    issue_at<K0, K1>(gtile, lds_tile, wave, lane, lane_off(wave, lane));
   }
 };
 
