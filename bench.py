@@ -51,6 +51,26 @@ def event_time(fn, iters, torch):
     return start.elapsed_time(stop) / iters
 
 
+def gpu_max_clock_mhz(torch):
+    """Maximum engine clock of GPU 0 in MHz, from the device properties or, failing that, rocminfo."""
+    mhz = getattr(torch.cuda.get_device_properties(0), "clock_rate", 0) / 1e3
+    if mhz > 0:
+        return mhz
+    try:
+        import re
+        import subprocess
+        text = subprocess.run(["rocminfo"], capture_output=True, text=True, timeout=30).stdout
+        # agents are listed in order; take the first one whose device type is GPU
+        for agent in text.split("*******")[1:]:
+            if re.search(r"Device Type:\s+GPU", agent):
+                m = re.search(r"Max Clock Freq\. \(MHz\):\s+(\d+)", agent)
+                if m:
+                    return float(m.group(1))
+    except Exception:
+        pass
+    return None
+
+
 def cpu_baseline(cfg, torch, budget_s=12.0):
     """Times the fp32 oracle (forward + autograd backward) on a few (b,h) units of the workload."""
     from oracle import diff_attn_oracle as orc
@@ -188,7 +208,7 @@ def main():
         "bwd_tflops": f_bwd / (sum(kernels_ms[k] for k in kernels_ms if k.startswith("bwd")) * 1e-3) / 1e12,
         "kernels_ms": kernels_ms,
         "device": {"name": prop.name, "cus": prop.multi_processor_count,
-                   "clock_mhz": getattr(prop, "clock_rate", 0) / 1e3, "peak_fp16_tflops_used": PEAK_FP16_TFLOPS},
+                   "clock_mhz": gpu_max_clock_mhz(torch), "peak_fp16_tflops_used": PEAK_FP16_TFLOPS},
         "roofline": roofline,
     }
     if args.workload != "headline":
