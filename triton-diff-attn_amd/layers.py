@@ -4,6 +4,9 @@ import math
 import torch
 
 from kernel import _diff_attention
+# stock-PyTorch comparison lines under the names the reference's benchmark imports from this
+# module (src/benchmark.py:11-17); none of them is used by MultiheadDiffAttnKernel
+from baselines import MultiheadAttn, MultiheadDiffAttn, MultiheadFlashAttn, MultiheadFlashDiffAttn  # noqa: F401
 
 
 def MultiheadDiffAttnKernel(
