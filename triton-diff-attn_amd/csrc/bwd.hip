@@ -443,6 +443,9 @@ template <int D, int NWAVES>
 struct DqCfg {
   static constexpr int DV = 2 * D;
   static constexpr int NW = NWAVES;            // waves per workgroup, 32 query rows each
+  // waves per SIMD the register budget is sized for: the resident Q1, Q2, dX rows and the two dQ
+  // accumulators of a D = 128 wave do not fit 256 registers
+  static constexpr int OCC = (D == 128) ? 1 : 2;
   static constexpr int NT = NW * 64;
   static constexpr int BM = NW * 32;           // query rows per workgroup
   static constexpr int BN = (D <= 64) ? 64 : 32;  // keys per staged tile
@@ -456,7 +459,7 @@ struct DqCfg {
 // [keys x queries], so that a lane owns one query column: the row statistics are per-lane
 // scalars and dS^T in accumulator layout is directly the B operand of dQ^T = K^T dS^T.
 template <int D, int NWAVES>
-__global__ __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(DqCfg<D, NWAVES>::OCC, DqCfg<D, NWAVES>::OCC))) void bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<D, NWAVES>;
   constexpr int DV = C::DV, NW = C::NW, BM = C::BM, BN = C::BN;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
@@ -631,8 +634,9 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 8u) {
-    // 256 query rows per workgroup when the sequence allows it, otherwise 128
-    if (p.N % 256 == 0)
+    // 256 query rows per workgroup when the sequence allows it, otherwise 128; a D = 128 workgroup
+    // runs one wave per SIMD and therefore has four waves
+    if (p.N % 256 == 0 && D != 128)
       hipLaunchKernelGGL((bwd_dq_kernel<D, 8>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
     else
       hipLaunchKernelGGL((bwd_dq_kernel<D, 4>), dim3(p.BH * (p.N / 128)), dim3(256), 0, stream, p);

@@ -2,7 +2,7 @@
 // lambda-combine and RMSNorm epilogue.  Computes what the reference's forward kernel computes
 // (src/kernel.py:20-207) with a different decomposition:
 //
-//   * a workgroup of 8 waves owns 128 query rows; waves 0-3 run softmax stream 1 (Q1,K1) and
+//   * a workgroup of 8 waves owns 128 query rows (4 waves and 64 rows for D = 128); waves 0-3 run softmax stream 1 (Q1,K1) and
 //     waves 4-7 run stream 2 (Q2,K2) for the same rows, 32 rows per wave.  All 8 waves share
 //     the K1/K2/V tiles, double-buffered in LDS, and the two streams meet only in the epilogue;
 //   * scores are computed transposed, S^T = K * Q^T (K fragments from LDS as the MFMA A operand,
@@ -21,10 +21,12 @@ struct FwdCfg {
   static constexpr int DV = 2 * D;
   static constexpr int BN = (D <= 64) ? 64 : 32;   // keys per tile
   static constexpr int QS = 1;                     // 32-row query blocks per wave
-  static constexpr int BM = 128;                   // query rows per workgroup
+  // query rows per workgroup; the output accumulators of a D = 128 wave need more than 256
+  // registers, so those workgroups have four waves at one wave per SIMD
+  static constexpr int BM = (D == 128) ? 64 : 128;
   static constexpr int NW = 2 * BM / (32 * QS);    // waves per workgroup: half of them per softmax stream
   static constexpr int NT = NW * 64;
-  static constexpr int OCC = (QS == 2) ? 1 : 2;    // waves per SIMD the register budget is sized for
+  static constexpr int OCC = (QS == 2 || D == 128) ? 1 : 2;   // waves per SIMD the register budget is sized for
   static constexpr int K_TILE = BN * D;            // halfs, one stream (swizzled, unpadded)
   static constexpr int V_TILE = BN * DV;
   static constexpr int K_BUF = 2 * K_TILE;         // K1 and K2 of one tile
@@ -349,7 +351,7 @@ static hipError_t launch_fwd_t(const FwdParams& p, hipStream_t stream) {
 }
 
 // Tile-size choice per head dimension (replaces the reference's run-time autotuner,
-// src/kernel.py:12-19): 128 query rows per workgroup; 64 keys per step for D <= 64, 32 for D = 128.
+// src/kernel.py:12-19): 128 query rows per workgroup and 64 keys per step for D <= 64; 64 rows and 32 keys for D = 128.
 hipError_t launch_fwd(const FwdParams& p, int D, hipStream_t stream) {
   switch (D) {
     case 32:  return launch_fwd_t<32>(p, stream);
