@@ -1,0 +1,44 @@
+"""Compiles the backward kernels to gfx950 assembly (no GPU needed) and checks that no inline-assembly
+MFMA reads a register that a VALU instruction wrote immediately before it (see isa_scan.py)."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+import isa_scan
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "triton-diff-attn_amd", "csrc")
+
+
+def test_scanner_flags_a_write_right_before_an_asm_mfma():
+    bad = """
+\tv_accvgpr_write_b32 a67, v137
+\t;;#ASMSTART
+\tv_mfma_f32_32x32x16_f16 v[18:33], v[66:69], a[64:67], v[18:33]
+\t;;#ASMEND
+"""
+    assert len(isa_scan.asm_mfma_hazards(bad)) == 1
+    spaced = bad.replace("\t;;#ASMSTART", "\ts_nop 2\n\t;;#ASMSTART")
+    assert isa_scan.asm_mfma_hazards(spaced) == []
+    # a compiler-visible MFMA is the compiler's business; an LDS load is ordered by s_waitcnt
+    assert isa_scan.asm_mfma_hazards(bad.replace("\t;;#ASMSTART\n", "").replace("\t;;#ASMEND\n", "")) == []
+    assert isa_scan.asm_mfma_hazards(bad.replace("v_accvgpr_write_b32 a67, v137", "ds_read_b128 v[66:69], v1")) == []
+    assert isa_scan.registers("v[2:4], a7, s[0:1], v10") == {"v2", "v3", "v4", "a7", "v10"}
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_backward_kernels_have_no_unprotected_asm_mfma(tmp_path):
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("da_build", os.path.join(ROOT, "triton-diff-attn_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    out = tmp_path / "bwd.s"
+    cmd = [build.HIPCC] + [f for f in build.FLAGS if f != "-fPIC"] + ["--cuda-device-only", "-S", "-o", str(out),
+                                                                          os.path.join(CSRC, "bwd.hip")]
+    subprocess.run(cmd, check=True, capture_output=True)
+    text = out.read_text()
+    assert "v_mfma_f32_32x32x16_f16" in text and ";;#ASMSTART" in text
+    hazards = isa_scan.asm_mfma_hazards(text)
+    assert hazards == [], "VALU write right before an inline-asm MFMA: %s" % hazards[:5]

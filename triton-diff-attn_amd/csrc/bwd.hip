@@ -132,11 +132,15 @@ struct DkvCfg {
 // dK_t and dV for one block of keys.  Products are formed as [queries x keys] so that a lane owns
 // one key column; P and dS in accumulator layout are then directly the A operands (rows = keys,
 // contraction over queries) of dV = P^T dX and dK_t = dS_t^T Q_t.
-template <int D>
+// MODE 0 computes dV, dK1 and dK2 in one pass.  At D = 128 their accumulators plus the resident
+// K1, K2, V rows exceed the 512 registers of a lane, so the work is split in two launches:
+// MODE 1 computes dV only (scores S1, S2; no dP), MODE 2 computes dK1 and dK2 only.
+template <int D, int MODE>
 __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_kernel(BwdParams p) {
   using C = DkvCfg<D>;
   constexpr int DV = C::DV, NW = C::NW, BK = C::BK, BQ = C::BQ;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32, NVT = DV / 32;
+  constexpr bool DO_V = (MODE != 2), DO_K = (MODE != 1);
 
   __shared__ __attribute__((aligned(16))) half_t smem[C::NBUF * C::STAGE];
 
@@ -169,8 +173,16 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
       for (int e = 0; e < 8; ++e) { x1[e] = (half_t)((float)x1[e] * c); x2[e] = (half_t)((float)x2[e] * c); }
       kf1[ks] = x1; kf2[ks] = x2;
     }
+    if constexpr (DO_K) {
 #pragma unroll
-    for (int kv = 0; kv < NKV; ++kv) vf[kv] = *reinterpret_cast<const h8*>(rv + 16 * kv);
+      for (int kv = 0; kv < NKV; ++kv) vf[kv] = *reinterpret_cast<const h8*>(rv + 16 * kv);
+    }
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) { keep_in_agpr(kf1[ks]); keep_in_agpr(kf2[ks]); }
+    if constexpr (DO_K) {
+#pragma unroll
+      for (int kv = 0; kv < NKV; ++kv) keep_in_agpr(vf[kv]);
+    }
   }
 
   f16v dv[NVT], dk1[NDT], dk2[NDT];
@@ -223,26 +235,24 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   constexpr int SPT = BQ / 32;
   struct Scores { f16v s1, s2, dp; };
   struct Packed { h8 pc[2], d1[2], d2[2]; };   // A operands of the dV / dK1 / dK2 products
-  constexpr int NPROD = 2 * NKS + NKV;         // matrix products per sub-tile in the first phase
+  constexpr int NPROD = 2 * NKS + (DO_K ? NKV : 0);   // score products per sub-tile (dP is needed for dK only)
   constexpr int DEPTH = 3;                     // A fragments requested ahead of their product
 
-  // Product k of a sub-tile: even k is k-step k/2 of dP; odd k alternates k-steps of S1 and S2.
-  // Two products of one chain are never neighbours: a product whose accumulator input is the
-  // result of the product issued just before the previous one was observed to read stale values
-  // when the one in between writes AGPRs.
+  // Product k of a sub-tile: even k is k-step k/2 of dP, odd k alternates k-steps of S1 and S2, so
+  // the three accumulation chains advance together; without dP (MODE 1) S1 and S2 alternate.
   static_assert(NKV == 2 * NKS, "every second product belongs to dP");
   auto prod_frag = [&](int buf, int qs, int k) -> h8 {
     const half_t* sQ1 = smem + buf * C::STAGE;
-    if (k & 1) {
-      const int t = k >> 1;
+    if (!DO_K || (k & 1)) {
+      const int t = DO_K ? (k >> 1) : k;
       const half_t* sQ = sQ1 + (t & 1) * C::Q_TILE;
       return *reinterpret_cast<const h8*>(sQ + swz_off<D>(qs * 32 + j, 16 * (t >> 1) + 8 * g));
     }
     return *reinterpret_cast<const h8*>(sQ1 + 2 * C::Q_TILE + swz_off<DV>(qs * 32 + j, 16 * (k >> 1) + 8 * g));
   };
   auto prod_mfma = [&](int k, h8 a, Scores& out) {
-    if (k & 1) {
-      const int t = k >> 1, ks = t >> 1;
+    if (!DO_K || (k & 1)) {
+      const int t = DO_K ? (k >> 1) : k, ks = t >> 1;
       if (t & 1) out.s2 = mfma32_bagpr(a, kf2[ks], out.s2);
       else       out.s1 = mfma32_bagpr(a, kf1[ks], out.s1);
     } else {
@@ -256,12 +266,21 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     const float* sStat = reinterpret_cast<const float*>(smem + buf * C::STAGE + 2 * C::Q_TILE + C::X_TILE);
     return *reinterpret_cast<const f4v*>(sStat + which * BQ + qs * 32 + 8 * r4 + 4 * g);
   };
+  auto results_ready = [&](Scores& s) {
+    if constexpr (DO_K) mfma_results_ready(s.s1, s.s2, s.dp);
+    else mfma_results_ready(s.s1, s.s2);
+  };
   auto init_scores = [&](int buf, int qs, Scores& out) {
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
-      const f4v a = stat4(buf, qs, 0, r4), bq = stat4(buf, qs, 1, r4), cq = stat4(buf, qs, 2, r4);
+      const f4v a = stat4(buf, qs, 0, r4), bq = stat4(buf, qs, 1, r4);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) { out.s1[4 * r4 + e] = a[e]; out.s2[4 * r4 + e] = bq[e]; out.dp[4 * r4 + e] = cq[e]; }
+      for (int e = 0; e < 4; ++e) { out.s1[4 * r4 + e] = a[e]; out.s2[4 * r4 + e] = bq[e]; }
+      if constexpr (DO_K) {
+        const f4v cq = stat4(buf, qs, 2, r4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out.dp[4 * r4 + e] = cq[e];
+      }
     }
   };
   // Element-wise work of accumulator register r (query row 8*(r/4) + 4g + (r%4)), split in three
@@ -271,19 +290,29 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   auto ew1 = [&](int r, const f4v& st3, const Scores& in, RowTmp& t) {
     t.p1[r] = fast_exp2(in.s1[r]);
     t.p2[r] = fast_exp2(in.s2[r]);
-    t.u[r] = __builtin_fmaf(-lam, in.dp[r], st3[r % 4]);
-    asm volatile("" : "+v"(t.p1[r]), "+v"(t.p2[r]), "+v"(t.u[r]));   // computed here, not moved to its use
+    if constexpr (DO_K) {
+      t.u[r] = __builtin_fmaf(-lam, in.dp[r], st3[r % 4]);
+      asm volatile("" : "+v"(t.p1[r]), "+v"(t.p2[r]), "+v"(t.u[r]));   // computed here, not moved to its use
+    } else {
+      asm volatile("" : "+v"(t.p1[r]), "+v"(t.p2[r]));
+    }
   };
   auto ew2 = [&](int r, const Scores& in, RowTmp& t) {
-    t.ds1[r] = t.p1[r] * in.dp[r];
-    t.ds2[r] = t.p2[r] * t.u[r];
-    t.pc[r] = __builtin_fmaf(-lam, t.p2[r], t.p1[r]);
-    asm volatile("" : "+v"(t.ds1[r]), "+v"(t.ds2[r]), "+v"(t.pc[r]));
+    if constexpr (DO_K) {
+      t.ds1[r] = t.p1[r] * in.dp[r];
+      t.ds2[r] = t.p2[r] * t.u[r];
+    }
+    if constexpr (DO_V) t.pc[r] = __builtin_fmaf(-lam, t.p2[r], t.p1[r]);
+    if constexpr (DO_K && DO_V) asm volatile("" : "+v"(t.ds1[r]), "+v"(t.ds2[r]), "+v"(t.pc[r]));
+    else if constexpr (DO_K) asm volatile("" : "+v"(t.ds1[r]), "+v"(t.ds2[r]));
+    else asm volatile("" : "+v"(t.pc[r]));
   };
   auto ew3 = [&](int r, const RowTmp& t, Packed& out) {   // r odd: packs rows r-1 and r
-    out.pc[r / 8][r % 8 - 1] = (half_t)t.pc[r - 1]; out.pc[r / 8][r % 8] = (half_t)t.pc[r];
-    out.d1[r / 8][r % 8 - 1] = (half_t)t.ds1[r - 1]; out.d1[r / 8][r % 8] = (half_t)t.ds1[r];
-    out.d2[r / 8][r % 8 - 1] = (half_t)t.ds2[r - 1]; out.d2[r / 8][r % 8] = (half_t)t.ds2[r];
+    if constexpr (DO_V) { out.pc[r / 8][r % 8 - 1] = (half_t)t.pc[r - 1]; out.pc[r / 8][r % 8] = (half_t)t.pc[r]; }
+    if constexpr (DO_K) {
+      out.d1[r / 8][r % 8 - 1] = (half_t)t.ds1[r - 1]; out.d1[r / 8][r % 8] = (half_t)t.ds1[r];
+      out.d2[r / 8][r % 8 - 1] = (half_t)t.ds2[r - 1]; out.d2[r / 8][r % 8] = (half_t)t.ds2[r];
+    }
   };
   // slot s of the skewed schedule: stage 1 of row s, stage 2 of row s-1, stage 3 of the pair ending at row s-2
   auto ew_slot = [&](int s, const f4v (&st)[4], const Scores& in, RowTmp& t, Packed& out) {
@@ -291,28 +320,31 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     if (s >= 1 && s - 1 < 16) ew2(s - 1, in, t);
     if (s >= 2 && s - 2 < 16 && ((s - 2) & 1)) ew3(s - 2, t, out);
   };
-  // B fragment (transposing read) of accumulate product m of sub-tile qs: m = kk*(NVT+2*NDT) + slot
-  constexpr int NACC1 = NVT + 2 * NDT;         // products per 16-query k-step
+  // B fragment (transposing read) of accumulate product m of sub-tile qs: m = kk*NACC1 + slot, where
+  // the slots of a 16-query k-step are the dV feature tiles followed by the dK1/dK2 feature tiles
+  constexpr int NSV = DO_V ? NVT : 0;          // dV slots
+  constexpr int NACC1 = NSV + (DO_K ? 2 * NDT : 0);
   constexpr int NACC = 2 * NACC1;
-  static_assert(NACC == NPROD, "one accumulate product per score product");
+  static_assert(NPROD % NACC == 0, "a whole number of score products per accumulate product");
+  constexpr int RATIO = NPROD / NACC;
   auto acc_frag = [&](int buf, int qs, int m) -> h8 {
     const half_t* sQ1 = smem + buf * C::STAGE;
     const int kk = m / NACC1, slot = m % NACC1;
     const int rbase = qs * 32 + 16 * kk + tr_row;
-    if (slot < NVT) {
+    if (slot < NSV) {
       const half_t* sX = sQ1 + 2 * C::Q_TILE;
       return join(lds_read_tr(sX + swz_off<DV>(rbase, 32 * slot + tr_col)),
                   lds_read_tr(sX + swz_off<DV>(rbase + 8, 32 * slot + tr_col)));
     }
-    const int t2 = slot - NVT;
+    const int t2 = slot - NSV;
     const half_t* sQ = sQ1 + (t2 & 1) * C::Q_TILE;
     return join(lds_read_tr(sQ + swz_off<D>(rbase, 32 * (t2 >> 1) + tr_col)),
                 lds_read_tr(sQ + swz_off<D>(rbase + 8, 32 * (t2 >> 1) + tr_col)));
   };
   auto acc_mfma = [&](int m, h8 bfrag, const Packed& in) {
     const int kk = m / NACC1, slot = m % NACC1;
-    if (slot < NVT) { dv[slot] = mfma32(in.pc[kk], bfrag, dv[slot]); return; }
-    const int t2 = slot - NVT;
+    if (slot < NSV) { dv[slot] = mfma32(in.pc[kk], bfrag, dv[slot]); return; }
+    const int t2 = slot - NSV;
     if (t2 & 1) dk2[t2 >> 1] = mfma32(in.d2[kk], bfrag, dk2[t2 >> 1]);
     else        dk1[t2 >> 1] = mfma32(in.d1[kk], bfrag, dk1[t2 >> 1]);
   };
@@ -321,10 +353,10 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   const int n_sub = p.N / 32;
   auto buf_of = [](int tile) { return tile % C::NBUF; };
 
-  // One step.  Chunk k holds score product k of sub-tile (bufn, qsn), accumulate product
-  // (k + NACC/2) % NACC -- the upper query half of sub-tile (bufp, qsp) while k < NACC/2, then the
-  // lower query half of sub-tile (bufc, qsc) -- and its share of the element-wise rows of sub-tile
-  // (bufc, qsc).  `pk` holds the packed operands: its lower half is written during the first half
+  // One step.  Chunk k holds score product k of sub-tile (bufn, qsn), every RATIO-th chunk also
+  // accumulate product (k/RATIO + NACC/2) % NACC -- the upper query half of sub-tile (bufp, qsp)
+  // during the first half of the step, then the lower query half of sub-tile (bufc, qsc) -- and
+  // every chunk its share of the element-wise rows of sub-tile (bufc, qsc).  `pk` holds the packed operands: its lower half is written during the first half
   // of the step and read during the second, its upper half is written during the second half and
   // read during the first half of the next step.
   static_assert(NPROD % 16 == 0 || 16 % NPROD == 0, "rows are spread evenly over the products");
@@ -335,9 +367,9 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     constexpr int LEAD = 2;                    // slots run before the first product
     // rows 0..7 are packed by slot 9, which must precede the first product that reads them
     static_assert(LEAD + (NSLOT - LEAD) * (NPROD / 2) / NPROD > 9, "lower half packed before it is read");
-    auto bfrag = [&](int k) -> h8 {
-      const int m = (k + NACC / 2) % NACC;
-      return (k < NACC / 2) ? acc_frag(bufp, qsp, m) : acc_frag(bufc, qsc, m);
+    auto bfrag = [&](int ja) -> h8 {
+      const int m = (ja + NACC / 2) % NACC;
+      return (ja < NACC / 2) ? acc_frag(bufp, qsp, m) : acc_frag(bufc, qsc, m);
     };
     h8 a[NPROD], bf[NACC];
     f4v st[4];
@@ -345,7 +377,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     init_scores(bufn, qsn, s_nxt);
 #pragma unroll
     for (int k = 0; k < DEPTH; ++k) a[k] = prod_frag(bufn, qsn, k);
-    st[0] = stat4(bufc, qsc, 3, 0);
+    if constexpr (DO_K) st[0] = stat4(bufc, qsc, 3, 0);
 #pragma unroll
     for (int k = 0; k < AHEAD; ++k) bf[k] = bfrag(k);
     // the first slots run while the initial accumulator values and the first fragments arrive
@@ -355,13 +387,13 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
 #pragma unroll
     for (int k = 0; k < NPROD; ++k) {
       if (k + DEPTH < NPROD) a[k + DEPTH] = prod_frag(bufn, qsn, k + DEPTH);
-      if (k + AHEAD < NACC) bf[k + AHEAD] = bfrag(k + AHEAD);
+      if (k % RATIO == 0 && k / RATIO + AHEAD < NACC) bf[k / RATIO + AHEAD] = bfrag(k / RATIO + AHEAD);
       // statistics of the next row group, requested a quarter of a step ahead of their use
-      if (k % (NPROD / 4) == 0 && k / (NPROD / 4) < 3) st[k / (NPROD / 4) + 1] = stat4(bufc, qsc, 3, k / (NPROD / 4) + 1);
+      if (DO_K && k % (NPROD / 4) == 0 && k / (NPROD / 4) < 3) st[k / (NPROD / 4) + 1] = stat4(bufc, qsc, 3, k / (NPROD / 4) + 1);
       // the next tile's fetch is spread over the products so that the waves do not queue up at the memory pipeline
       if (fetch && k % (NPROD / 4) == 1) stage(tile_next, buf_next, k / (NPROD / 4));
       prod_mfma(k, a[k], s_nxt);
-      acc_mfma((k + NACC / 2) % NACC, bf[k], pk);
+      if (k % RATIO == 0) acc_mfma((k / RATIO + NACC / 2) % NACC, bf[k / RATIO], pk);
       // slots LEAD .. NSLOT-1 spread over the products
       const int s0 = LEAD + (NSLOT - LEAD) * k / NPROD, s1 = LEAD + (NSLOT - LEAD) * (k + 1) / NPROD;
 #pragma unroll
@@ -369,7 +401,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
       __builtin_amdgcn_sched_barrier(0);
     }
     // the next step's VALU reads these results right away
-    mfma_results_ready(s_nxt.s1, s_nxt.s2, s_nxt.dp);
+    results_ready(s_nxt);
   };
 
   // step i: compile-time positions of sub-tiles i+1, i, i-1 inside their tiles
@@ -409,7 +441,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   init_scores(0, 0, sa);
 #pragma unroll
   for (int k = 0; k < NPROD; ++k) prod_mfma(k, prod_frag(0, 0, k), sa);
-  mfma_results_ready(sa.s1, sa.s2, sa.dp);
+  results_ready(sa);
 
   for (int i = 0; i < n_sub; i += 2) {   // the sub-tile count is even
     step(i, std::integral_constant<int, 1 % SPT>{}, sa, sb, pk);
@@ -421,21 +453,25 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
 
   // accumulator tile tt: column = 32*tt + j (feature), register r = key row 8*(r/4) + 4g + (r%4)
   const size_t krow0 = row0 + (size_t)kt * BK + wave * 32;
+  if constexpr (DO_V) {
 #pragma unroll
-  for (int tt = 0; tt < NVT; ++tt)
+    for (int tt = 0; tt < NVT; ++tt)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int kr = 8 * (r / 4) + 4 * g + (r % 4);
-      p.dv[(krow0 + kr) * DV + 32 * tt + j] = (half_t)dv[tt][r];
-    }
+      for (int r = 0; r < 16; ++r) {
+        const int kr = 8 * (r / 4) + 4 * g + (r % 4);
+        p.dv[(krow0 + kr) * DV + 32 * tt + j] = (half_t)dv[tt][r];
+      }
+  }
+  if constexpr (DO_K) {
 #pragma unroll
-  for (int tt = 0; tt < NDT; ++tt)
+    for (int tt = 0; tt < NDT; ++tt)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int kr = 8 * (r / 4) + 4 * g + (r % 4);
-      p.dk1[(krow0 + kr) * D + 32 * tt + j] = (half_t)(dk1[tt][r] * p.sm_scale);
-      p.dk2[(krow0 + kr) * D + 32 * tt + j] = (half_t)(dk2[tt][r] * p.sm_scale);
-    }
+      for (int r = 0; r < 16; ++r) {
+        const int kr = 8 * (r / 4) + 4 * g + (r % 4);
+        p.dk1[(krow0 + kr) * D + 32 * tt + j] = (half_t)(dk1[tt][r] * p.sm_scale);
+        p.dk2[(krow0 + kr) * D + 32 * tt + j] = (half_t)(dk2[tt][r] * p.sm_scale);
+      }
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -630,7 +666,14 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 4u) {
-    hipLaunchKernelGGL((bwd_dkdv_kernel<D>), dim3(p.BH * (p.N / DkvCfg<D>::BK)), dim3(DkvCfg<D>::NT), 0, stream, p);
+    const dim3 grid(p.BH * (p.N / DkvCfg<D>::BK)), block(DkvCfg<D>::NT);
+    if constexpr (D == 128) {
+      hipLaunchKernelGGL((bwd_dkdv_kernel<D, 1>), grid, block, 0, stream, p);
+      if ((e = hipGetLastError()) != hipSuccess) return e;
+      hipLaunchKernelGGL((bwd_dkdv_kernel<D, 2>), grid, block, 0, stream, p);
+    } else {
+      hipLaunchKernelGGL((bwd_dkdv_kernel<D, 0>), grid, block, 0, stream, p);
+    }
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 8u) {

@@ -47,9 +47,18 @@ __device__ __forceinline__ f16v mfma32_bagpr(h8 a, h8 b, f16v c) {
   asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
   return c;
 }
+// Moves a fragment into AGPRs for good: after this the value is defined by an (empty) asm statement
+// with an AGPR output, so the compiler has no VGPR original to copy from in front of a later use.
+// A v_accvgpr_write directly in front of an inline-asm MFMA that reads the AGPR is a hazard the
+// compiler covers for its own MFMAs only: the MFMA was observed to read the old register content.
+__device__ __forceinline__ void keep_in_agpr(h8& x) { asm volatile("" : "+a"(x)); }
+
 // Wait states that cover the write-back of an 8-pass MFMA before a VALU instruction reads it.
 __device__ __forceinline__ void mfma_results_ready(f16v& x, f16v& y, f16v& z) {
   asm volatile("s_nop 15\n\ts_nop 3" : "+v"(x), "+v"(y), "+v"(z));
+}
+__device__ __forceinline__ void mfma_results_ready(f16v& x, f16v& y) {
+  asm volatile("s_nop 15\n\ts_nop 3" : "+v"(x), "+v"(y));
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
