@@ -1,0 +1,73 @@
+"""The differential-attention layer (modules.py): host-side structure on the CPU with the stock-PyTorch
+operator plugged in, and on the GPU the same layer with the fused kernel against the stock operator."""
+import copy
+import math
+
+import pytest
+import torch
+
+import baselines
+import modules
+
+
+def test_lambda_schedule_and_reparametrisation():
+    assert modules.lambda_init_for_depth(0) == pytest.approx(0.2)
+    assert modules.lambda_init_for_depth(10) == pytest.approx(0.8 - 0.6 * math.exp(-3.0))
+    layer = modules.DiffAttn(64, 2, depth=3, attention=baselines.MultiheadDiffAttn, dtype=torch.float32)
+    with torch.no_grad():
+        layer.lambda_q1.fill_(0.5); layer.lambda_k1.fill_(0.25); layer.lambda_q2.fill_(-0.5); layer.lambda_k2.fill_(0.5)
+    d = layer.head_dim
+    want = math.exp(0.125 * d) - math.exp(-0.25 * d) + layer.lambda_init
+    assert layer.lambda_scale().shape == (1,)
+    assert layer.lambda_scale().item() == pytest.approx(want, rel=1e-5)
+
+
+def test_layer_shapes_and_gradients_reach_every_parameter():
+    torch.manual_seed(0)
+    layer = modules.DiffAttn(64, 2, depth=1, attention=baselines.MultiheadDiffAttn, dtype=torch.float32)
+    assert layer.head_dim == 16
+    x = torch.randn(2, 24, 64, requires_grad=True)
+    y = layer(x)
+    assert y.shape == x.shape
+    y.square().mean().backward()
+    for name, p in layer.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all() and p.grad.abs().sum() > 0, name
+    assert x.grad is not None
+    with pytest.raises(ValueError):
+        modules.DiffAttn(60, 4)
+
+
+def test_layer_matches_a_direct_evaluation_of_its_formula():
+    torch.manual_seed(1)
+    layer = modules.DiffAttn(32, 2, depth=2, attention=baselines.MultiheadDiffAttn, dtype=torch.float32)
+    x = torch.randn(1, 8, 32)
+    B, N, E, H, d = 1, 8, 32, 2, 8
+    q = layer.q_proj(x).view(B, N, 2 * H, d).transpose(1, 2)
+    k = layer.k_proj(x).view(B, N, 2 * H, d).transpose(1, 2)
+    v = layer.v_proj(x).view(B, N, H, 2 * d).transpose(1, 2)
+    a = torch.softmax(q @ k.transpose(-1, -2) / math.sqrt(d), -1).view(B, H, 2, N, N)
+    lam = layer.lambda_scale()
+    heads = (a[:, :, 0] - lam * a[:, :, 1]) @ v
+    heads = heads * torch.rsqrt(heads.square().mean(-1, keepdim=True) + 1e-5) * (1 - layer.lambda_init) * layer.head_gain
+    want = layer.out_proj(heads.transpose(1, 2).reshape(B, N, E))
+    assert torch.allclose(layer(x), want, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_layer_with_the_kernel_matches_the_stock_operator():
+    torch.manual_seed(2)
+    dev = torch.device("cuda:0")
+    fused = modules.DiffAttn(512, 4, depth=2, device=dev)            # head_dim 64, fp16
+    stock = copy.deepcopy(fused)
+    stock.attention = baselines.MultiheadDiffAttn
+    x = (0.5 * torch.randn(2, 256, 512, device=dev)).half()
+    xs = [x.clone().requires_grad_(True) for _ in range(2)]
+    ys = [m(xi) for m, xi in zip((fused, stock), xs)]
+    assert (ys[0].float() - ys[1].float()).abs().max().item() <= 1e-2
+    g = torch.randn_like(ys[0])
+    for y in ys:
+        y.backward(g)
+    assert (xs[0].grad.float() - xs[1].grad.float()).abs().max().item() <= 2e-2 * xs[1].grad.float().abs().max().item() + 1e-3
+    for (name, pf), (_, ps) in zip(fused.named_parameters(), stock.named_parameters()):
+        scale = ps.grad.float().abs().max().item()
+        assert (pf.grad.float() - ps.grad.float()).abs().max().item() <= 5e-2 * scale + 1e-3, name
