@@ -30,11 +30,16 @@ WORKLOADS = {
     "headline": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0),
     "config1": dict(B=2, H=16, N=512, D=32, lam=0.5, lambda_init=0.8, rms=True, seed=0, scale=1.0),
     "config4": dict(B=8, H=32, N=4096, D=128, lam=0.8, lambda_init=0.2, rms=False, seed=4, scale=1.0),
+    # the headline shape with the causal mask (an addition to the reference's operator)
+    "headline_causal": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0, causal=True),
 }
 
 
 def flops(cfg):
-    unit = cfg["B"] * cfg["H"] * cfg["N"] ** 2 * cfg["D"]
+    """Algorithmic matmul FLOPs (forward, backward); with the causal mask only the N(N+1)/2 visible
+    (query, key) pairs count."""
+    pairs = cfg["N"] * (cfg["N"] + 1) // 2 if cfg.get("causal") else cfg["N"] ** 2
+    unit = cfg["B"] * cfg["H"] * pairs * cfg["D"]
     return 12 * unit, 20 * unit
 
 
@@ -83,7 +88,8 @@ def cpu_baseline(cfg, torch, budget_s=12.0):
     units = 8
     q1, q2, k1, k2, v, dy = make_inputs(1, units, N, D, cfg["seed"], cfg["scale"])
     lam = torch.tensor([cfg["lam"]], dtype=torch.float16)
-    run = lambda: orc.forward_backward(q1, q2, k1, k2, v, lam, dy, cfg["lambda_init"], cfg["rms"], chunk=1)
+    run = lambda: orc.forward_backward(q1, q2, k1, k2, v, lam, dy, cfg["lambda_init"], cfg["rms"], chunk=1,
+                                       causal=bool(cfg.get("causal")))
     run()  # warm-up
     t0 = time.perf_counter()
     reps = 0
@@ -93,7 +99,7 @@ def cpu_baseline(cfg, torch, budget_s=12.0):
         if time.perf_counter() - t0 > budget_s or reps >= 200:
             break
     dt = (time.perf_counter() - t0) / reps
-    fl = 32.0 * units * N * N * D
+    fl = float(sum(flops(dict(cfg, B=1, H=units))))
     return {
         "value": fl / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
         "sample": "%d of %d (batch,head) units of the workload, fp32 oracle forward+autograd backward, %d repetitions, "
@@ -133,7 +139,8 @@ def main():
         for t in leaves:
             t.grad = None
         lam.grad = None
-        y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"])
+        y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"],
+                                    causal=bool(cfg.get("causal")))
         y.backward(dy)
 
     for _ in range(args.warmup):
@@ -158,19 +165,20 @@ def main():
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream().cuda_stream
         sm = 1 / math.sqrt(D)
+        flags = int(cfg["rms"]) | (2 if cfg.get("causal") else 0)     # DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL
 
         def fwd_only():
             _native.check(lib.diffattn_forward(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(),
-                B, H, N, D, sm, cfg["lambda_init"], int(cfg["rms"]), stream))
+                B, H, N, D, sm, cfg["lambda_init"], flags, stream))
 
         def bwd_stage(mask):
             return lambda: _native.check(lib.diffattn_backward_stages(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(), dy.data_ptr(),
                 *[g.data_ptr() for g in grads], dlam.data_ptr(), ws.data_ptr(), ws_bytes,
-                B, H, N, D, sm, cfg["lambda_init"], int(cfg["rms"]), mask, stream))
+                B, H, N, D, sm, cfg["lambda_init"], flags, mask, stream))
 
         fwd_only(); bwd_stage(15)()
         k_iters = max(5, min(args.steps, 30))
@@ -181,7 +189,7 @@ def main():
             "bwd_dkdv_kernel": event_time(bwd_stage(4), k_iters, torch),
             "bwd_dq_kernel": event_time(bwd_stage(8), k_iters, torch),
         }
-    unit = B * H * N * N * D
+    unit = f_fwd // 12
     dkdv_flops = 16 * unit      # S1,S2 (4) + dP (4) + dV (4) + dK1,dK2 (4), times B*H*N^2*D
     dkdv_tflops = dkdv_flops / (kernels_ms["bwd_dkdv_kernel"] * 1e-3) / 1e12
     traffic = None
@@ -202,7 +210,8 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "%s: diff-attn fwd+bwd B%d H%d N%d D%d fp16 rms_norm=%s lambda=%.1f lambda_init=%.1f"
-                               % (args.workload, B, H, N, D, cfg["rms"], cfg["lam"], cfg["lambda_init"])},
+                               % (args.workload, B, H, N, D, cfg["rms"], cfg["lam"], cfg["lambda_init"])
+                               + (" causal" if cfg.get("causal") else "")},
         "frac_of_fp16_mfma_peak": value / PEAK_FP16_TFLOPS,
         "fwd_tflops": f_fwd / (kernels_ms["fwd_kernel"] * 1e-3) / 1e12,
         "bwd_tflops": f_bwd / (sum(kernels_ms[k] for k in kernels_ms if k.startswith("bwd")) * 1e-3) / 1e12,

@@ -33,6 +33,15 @@ extern "C" {
 #define DIFFATTN_EINVAL_SEQ (-3)    /* N not a multiple of 128 */
 #define DIFFATTN_EINVAL_WS (-4)     /* workspace too small */
 #define DIFFATTN_EINVAL_ALIGN (-5)  /* a pointer is not 16-byte aligned */
+#define DIFFATTN_EINVAL_FLAGS (-6)  /* unknown bits in `flags` */
+
+/* `flags` of the forward and backward entry points.  DIFFATTN_RMS_NORM is the reference's boolean
+ * `rms_norm` (src/kernel.py:464): a caller that passes a C boolean there keeps working.
+ * DIFFATTN_CAUSAL has no counterpart in the reference, which lists masking as missing
+ * (src/kernel.py:4): query i sees keys 0..i only, in both softmax streams.  Forward and backward of
+ * one problem must be given the same flags. */
+#define DIFFATTN_RMS_NORM 1
+#define DIFFATTN_CAUSAL 2
 
 /* ABI version of this header; bumped when a signature changes. */
 int diffattn_abi_version(void);
@@ -42,18 +51,18 @@ const char* diffattn_strerror(int code);
 
 /*
  * Forward.  Replaces the launch of diff_attn_fwd (src/kernel.py:476-503).
- *   y    [B,H,N,2D]  out: (softmax(s q1 k1^T) - lambda softmax(s q2 k2^T)) v, then, iff rms_norm,
+ *   y    [B,H,N,2D]  out: (softmax(s q1 k1^T) - lambda softmax(s q2 k2^T)) v, then, iff DIFFATTN_RMS_NORM,
  *                    (1 - lambda_init) * rmsnorm(.) with eps 1e-5 (src/kernel.py:188-198)
  *   u2   [B,H,N,2D]  out, optional (may be NULL when no backward follows): softmax(s q2 k2^T) v
  *   lse1, lse2 [B,H,N] fp32 out, optional: natural-log row logsumexp of the scaled scores
  *                    (the reference's M1/M2, src/kernel.py:188-189,203-204)
- *   rinv [B,H,N] fp32 out, optional, written only when rms_norm: rsqrt(mean(x^2) + 1e-5)
+ *   rinv [B,H,N] fp32 out, optional, written only with DIFFATTN_RMS_NORM: rsqrt(mean(x^2) + 1e-5)
  * The reference additionally stores both per-stream outputs O1,O2 (src/kernel.py:205-206); here
  * the backward rebuilds the pre-norm row from y and rinv, so only u2 is kept.
  */
 int diffattn_forward(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
                      const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
-                     int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                     int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                      void* stream);
 
 /* Bytes of device workspace diffattn_backward needs for this problem size (0 on bad sizes). */
@@ -63,7 +72,7 @@ size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D);
  * Backward.  Replaces the launch of diff_attn_bwd (src/kernel.py:531-570) and the host-side
  * reduction of the lambda gradient (src/kernel.py:573).
  *   inputs : q1,q2,k1,k2,v,lambda_scale as in forward; y,u2,lse1,lse2,rinv as written by forward
- *            (rinv is ignored unless rms_norm); dy [B,H,N,2D] upstream gradient, dense.
+ *            (rinv is ignored without DIFFATTN_RMS_NORM); dy [B,H,N,2D] upstream gradient, dense.
  *   outputs: dq1,dq2,dk1,dk2 [B,H,N,D], dv [B,H,N,2D] fp16; dlambda: one fp16 value, DEVICE
  *            memory, written (not accumulated), reduced in a fixed order: bit-reproducible.
  *   workspace: device memory of at least diffattn_backward_workspace_bytes(B,H,N,D) bytes,
@@ -74,7 +83,7 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
                       const float* lse1, const float* lse2, const float* rinv, const void* dy,
                       void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                       void* workspace, size_t workspace_bytes,
-                      int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                      int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                       void* stream);
 
 /*
@@ -97,7 +106,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              const float* lse1, const float* lse2, const float* rinv, const void* dy,
                              void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                              void* workspace, size_t workspace_bytes,
-                             int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                             int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                              unsigned stage_mask, void* stream);
 
 #ifdef __cplusplus

@@ -33,16 +33,23 @@ def _as_scalar(lambda_scale, dtype):
     return torch.tensor(float(lambda_scale), dtype=dtype)
 
 
-def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False):
+def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False, causal=False):
     """One or more (b, h) units: tensors [..., N, D] / [..., N, 2D], already in the work dtype.
 
-    Follows src/layers.py:60-78 line for line (minus the .half() casts).
+    Follows src/layers.py:60-78 line for line (minus the .half() casts).  `causal` (not in the
+    reference, which lists masking as missing, src/kernel.py:4) lets query i see keys 0..i only, in
+    both softmax streams.
     """
     head_dim = q1.size(-1)
     sm_scale = 1 / math.sqrt(head_dim)                       # src/layers.py:60-62
     s1 = torch.matmul(q1, k1.transpose(-2, -1)) * sm_scale   # src/layers.py:64
-    p1 = torch.softmax(s1, dim=-1)                           # src/layers.py:65
     s2 = torch.matmul(q2, k2.transpose(-2, -1)) * sm_scale   # src/layers.py:67
+    if causal:
+        n = s1.size(-1)
+        future = torch.ones(n, n, dtype=torch.bool, device=s1.device).triu(1)
+        s1 = s1.masked_fill(future, float("-inf"))
+        s2 = s2.masked_fill(future, float("-inf"))
+    p1 = torch.softmax(s1, dim=-1)                           # src/layers.py:65
     p2 = torch.softmax(s2, dim=-1)                           # src/layers.py:68
     p = p1 - lam * p2                                        # src/layers.py:70
     x = torch.matmul(p, v)                                   # src/layers.py:72
@@ -66,7 +73,7 @@ def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False):
 
 
 def forward(q1, q2, k1, k2, v, lambda_scale, lambda_init=0.8, rms_norm=False,
-            dtype=torch.float32, chunk=8, want_aux=False):
+            dtype=torch.float32, chunk=8, want_aux=False, causal=False):
     """Differential attention forward, [B,H,N,D] inputs, result in `dtype`.
 
     Inputs are upcast (fp16 values are used exactly as rounded).  `chunk` = number of (b,h)
@@ -80,7 +87,7 @@ def forward(q1, q2, k1, k2, v, lambda_scale, lambda_init=0.8, rms_norm=False,
     ys, auxs = [], []
     for s in range(0, B * H, chunk):
         sl = slice(s, s + chunk)
-        r = forward_unit(q1f[sl], q2f[sl], k1f[sl], k2f[sl], vf[sl], lam, lambda_init, rms_norm, want_aux)
+        r = forward_unit(q1f[sl], q2f[sl], k1f[sl], k2f[sl], vf[sl], lam, lambda_init, rms_norm, want_aux, causal)
         if want_aux:
             ys.append(r[0]); auxs.append(r[1])
         else:
@@ -99,7 +106,7 @@ def forward(q1, q2, k1, k2, v, lambda_scale, lambda_init=0.8, rms_norm=False,
 
 
 def forward_backward(q1, q2, k1, k2, v, lambda_scale, dy, lambda_init=0.8, rms_norm=False,
-                     dtype=torch.float32, chunk=8):
+                     dtype=torch.float32, chunk=8, causal=False):
     """Forward + autograd backward of the restated graph.
 
     Returns (y, dq1, dq2, dk1, dk2, dv, dlambda) in `dtype`; dlambda has shape [1] and is the sum
@@ -119,7 +126,7 @@ def forward_backward(q1, q2, k1, k2, v, lambda_scale, dy, lambda_init=0.8, rms_n
         sl = slice(s, s + chunk)
         leaves = [t[sl].detach().clone().requires_grad_(True) for t in ins]
         lam = lam0.detach().clone().requires_grad_(True)
-        y = forward_unit(*leaves, lam, lambda_init, rms_norm)
+        y = forward_unit(*leaves, lam, lambda_init, rms_norm, causal=causal)
         g = torch.autograd.grad(y, leaves + [lam], dyf[sl])
         for dst, src in zip(grads, g[:5]):
             dst[sl] = src

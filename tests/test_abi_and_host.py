@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_symbols():
         assert hasattr(lib, name), name
         assert name in _native.SYMBOLS, "binding table misses %s" % name
-    assert lib.diffattn_abi_version() == 1
+    assert lib.diffattn_abi_version() == 2
 
 
 def test_argument_rejection_needs_no_gpu():
@@ -46,6 +46,9 @@ def test_argument_rejection_needs_no_gpu():
     bad = args(1, 1, 128, 64)
     bad[0] = p + 2
     assert lib.diffattn_forward(*bad) == -5
+    bad = args(1, 1, 128, 64)
+    bad[-2] = 4                                   # unknown flag bit
+    assert lib.diffattn_forward(*bad) == -6
     assert lib.diffattn_backward_workspace_bytes(1, 1, 100, 64) == 0
     assert lib.diffattn_backward_workspace_bytes(1, 1, 128, 48) == 0
     need = lib.diffattn_backward_workspace_bytes(2, 3, 256, 64)
@@ -53,7 +56,9 @@ def test_argument_rejection_needs_no_gpu():
     assert need >= rows * 128 * 2 + 4 * rows * 4
     bargs = [p] * 5 + [p, p, p, p, p, p, p] + [p] * 6 + [p, need - 1, 2, 3, 256, 64, 0.125, 0.8, 1, None]
     assert lib.diffattn_backward(*bargs) == -4
-    for code in (0, -1, -2, -3, -4, -5):
+    bargs[19], bargs[-2] = need, 8
+    assert lib.diffattn_backward(*bargs) == -6
+    for code in (0, -1, -2, -3, -4, -5, -6):
         assert len(lib.diffattn_strerror(code)) > 0
 
 
@@ -81,10 +86,14 @@ def test_drop_in_signature_matches_reference():
     import layers
     from kernel import _diff_attention
     sig = inspect.signature(layers.MultiheadDiffAttnKernel)
-    assert list(sig.parameters) == ["q1", "q2", "k1", "k2", "v", "lambda_scale", "lambda_init", "rms_norm"]
+    # the reference's eight parameters in the reference's order; `causal` is an addition at the end
+    assert list(sig.parameters) == ["q1", "q2", "k1", "k2", "v", "lambda_scale", "lambda_init", "rms_norm", "causal"]
+    assert sig.parameters["causal"].default is False
     assert sig.parameters["lambda_scale"].default == -0.5
     assert sig.parameters["lambda_init"].default == 0.8
     assert sig.parameters["rms_norm"].default is False
     fsig = inspect.signature(_diff_attention.forward)
-    assert list(fsig.parameters) == ["ctx", "Q1", "Q2", "K1", "K2", "V", "SM_SCALE", "LAMBDA_SCALE", "LAMBDA_INIT", "rms_norm"]
+    assert list(fsig.parameters) == ["ctx", "Q1", "Q2", "K1", "K2", "V", "SM_SCALE", "LAMBDA_SCALE", "LAMBDA_INIT", "rms_norm",
+                                     "causal"]
+    assert fsig.parameters["causal"].default is False
     assert issubclass(_diff_attention, torch.autograd.Function)

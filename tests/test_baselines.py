@@ -85,3 +85,12 @@ def test_sweep_script_host_helpers():
     assert all(a.requires_grad and a.dtype == torch.float16 for a in args)
     args, kwargs, _ = mod.make_case(False, 2, 3, 16, 8, gen, "cpu")
     assert [tuple(a.shape) for a in args] == [(2, 3, 16, 16)] * 3 and kwargs == {}
+
+
+@pytest.mark.parametrize("fn", [baselines.MultiheadDiffAttn, baselines.MultiheadFlashDiffAttn])
+def test_causal_comparison_lines_follow_the_oracle(fn):
+    q1, q2, k1, k2, v = _case()
+    lam = torch.tensor([0.4], dtype=torch.float16)
+    ref = orc.forward(q1, q2, k1, k2, v, lam, 0.8, True, causal=True)
+    got = fn(q1, q2, k1, k2, v, lambda_scale=lam, lambda_init=0.8, rms_norm=True, causal=True)
+    assert max_abs(got.float(), ref) <= ATOL

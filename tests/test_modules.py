@@ -71,3 +71,18 @@ def test_layer_with_the_kernel_matches_the_stock_operator():
     for (name, pf), (_, ps) in zip(fused.named_parameters(), stock.named_parameters()):
         scale = ps.grad.float().abs().max().item()
         assert (pf.grad.float() - ps.grad.float()).abs().max().item() <= 5e-2 * scale + 1e-3, name
+
+
+@pytest.mark.gpu
+def test_causal_layer_with_the_kernel_matches_the_stock_operator():
+    torch.manual_seed(3)
+    dev = torch.device("cuda:0")
+    fused = modules.DiffAttn(256, 2, depth=1, causal=True, device=dev)
+    stock = copy.deepcopy(fused)
+    stock.attention = baselines.MultiheadDiffAttn
+    x = (0.5 * torch.randn(1, 384, 256, device=dev)).half()
+    y_f, y_s = fused(x), stock(x)
+    assert (y_f.float() - y_s.float()).abs().max().item() <= 1e-2
+    # a causal layer's output at position i does not change when later positions do
+    x2 = x.clone(); x2[:, 200:] = 0
+    assert (fused(x2)[:, :200].float() - y_f[:, :200].float()).abs().max().item() <= 2e-3

@@ -150,3 +150,35 @@ def test_chunking_and_dtype():
     lam = torch.tensor([0.5], dtype=torch.float16)
     c = orc.forward(q1, q2, k1, k2, v, lam, rms_norm=True)
     assert torch.allclose(a, c, atol=1e-6)
+
+
+# ---- causal variant (not in the reference; pinned the same way) ---------------------------------
+from util import make_inputs, max_abs  # noqa: E402
+
+def test_causal_lambda_zero_is_causal_sdpa():
+    q1, q2, k1, k2, v, _ = make_inputs(1, 2, 48, 16, 11)
+    y = orc.forward(q1, q2, k1, k2, v, 0.0, 0.8, False, causal=True)
+    ref = F.scaled_dot_product_attention(q1.float(), k1.float(), v.float(), is_causal=True)
+    assert max_abs(y, ref) < 2e-5
+    y = orc.forward(q1, q2, k1, k2, v, 0.0, 0.8, True, causal=True)
+    assert max_abs(y, 0.2 * F.rms_norm(ref, (32,), eps=1e-5)) < 2e-5
+
+
+def test_causal_prefix_property_and_first_row():
+    # row i of the causal result depends on rows 0..i only: truncating the sequence changes nothing before the cut
+    q1, q2, k1, k2, v, _ = make_inputs(1, 1, 40, 8, 12)
+    lam = torch.tensor([0.6], dtype=torch.float16)
+    full = orc.forward(q1, q2, k1, k2, v, lam, 0.8, False, causal=True)
+    cut = orc.forward(*(t[:, :, :17] for t in (q1, q2, k1, k2, v)), lam, 0.8, False, causal=True)
+    assert max_abs(full[:, :, :17], cut) < 1e-6
+    # query 0 sees key 0 only: X_0 = (1 - lambda) v_0
+    assert max_abs(full[:, :, 0], (1 - lam.float()) * v[:, :, 0].float()) < 1e-6
+
+
+def test_causal_gradients_do_not_flow_from_the_past_to_future_keys():
+    q1, q2, k1, k2, v, dy = make_inputs(1, 1, 24, 8, 13)
+    dy = dy.clone(); dy[:, :, 10:] = 0          # only rows 0..9 receive gradient
+    out = orc.forward_backward(q1, q2, k1, k2, v, 0.5, dy, 0.8, True, causal=True)
+    for g in (out[3], out[4], out[5]):          # dk1, dk2, dv of keys 10.. are exactly zero
+        assert g[:, :, 10:].abs().max().item() == 0.0
+    assert out[3][:, :, :10].abs().max().item() > 0

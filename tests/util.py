@@ -26,14 +26,15 @@ def rel_to_max(a, ref):
     return (a.float().cpu() - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
 
 
-def run_kernel(q1, q2, k1, k2, v, lam_value, lambda_init, rms_norm, dy=None, device="cuda"):
+def run_kernel(q1, q2, k1, k2, v, lam_value, lambda_init, rms_norm, dy=None, device="cuda", causal=False):
     """Runs layers.MultiheadDiffAttnKernel on the GPU; returns (y, grads or None) as CPU tensors."""
     from layers import MultiheadDiffAttnKernel
 
     need = dy is not None
     t = [x.to(device).requires_grad_(need) for x in (q1, q2, k1, k2, v)]
     lam = torch.tensor([lam_value], dtype=torch.float16, device=device, requires_grad=need)
-    y = MultiheadDiffAttnKernel(*t, lambda_scale=lam, lambda_init=lambda_init, rms_norm=rms_norm)
+    extra = {"causal": True} if causal else {}
+    y = MultiheadDiffAttnKernel(*t, lambda_scale=lam, lambda_init=lambda_init, rms_norm=rms_norm, **extra)
     grads = None
     if need:
         y.backward(dy.to(device))

@@ -27,9 +27,12 @@ def _rms(x: torch.Tensor) -> torch.Tensor:
     return F.rms_norm(x, (x.size(-1),), eps=RMS_EPS)
 
 
-def _probabilities(q: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
+def _probabilities(q: torch.Tensor, k: torch.Tensor, causal: bool = False) -> torch.Tensor:
     """softmax(q k^T / sqrt(d)) with the softmax in fp32 and the result back in the input dtype."""
     scores = (q @ k.transpose(-1, -2)) * (1.0 / math.sqrt(q.size(-1)))
+    if causal:
+        n = scores.size(-1)
+        scores = scores.masked_fill(torch.ones(n, n, dtype=torch.bool, device=scores.device).triu(1), float("-inf"))
     return torch.softmax(scores.float(), dim=-1).to(q.dtype)
 
 
@@ -38,8 +41,9 @@ def MultiheadAttn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, rms_norm: b
     return _rms(out) if rms_norm else out
 
 
-def MultiheadDiffAttn(q1, q2, k1, k2, v, lambda_scale=-0.5, lambda_init: float = 0.8, rms_norm: bool = False):
-    weights = _probabilities(q1, k1) - lambda_scale * _probabilities(q2, k2)
+def MultiheadDiffAttn(q1, q2, k1, k2, v, lambda_scale=-0.5, lambda_init: float = 0.8, rms_norm: bool = False,
+                      causal: bool = False):
+    weights = _probabilities(q1, k1, causal) - lambda_scale * _probabilities(q2, k2, causal)
     out = weights @ v
     if rms_norm:
         out = (1 - lambda_init) * _rms(out)
@@ -51,11 +55,12 @@ def MultiheadFlashAttn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, rms_no
     return _rms(out) if rms_norm else out
 
 
-def MultiheadFlashDiffAttn(q1, q2, k1, k2, v, lambda_scale=-0.5, lambda_init: float = 0.8, rms_norm: bool = False):
+def MultiheadFlashDiffAttn(q1, q2, k1, k2, v, lambda_scale=-0.5, lambda_init: float = 0.8, rms_norm: bool = False,
+                           causal: bool = False):
     # fused attention kernels want equal head dims for q, k and v: each stream runs once per half of v
     halves = v.split(q1.size(-1), dim=-1)
-    stream1 = torch.cat([F.scaled_dot_product_attention(q1, k1, h) for h in halves], dim=-1)
-    stream2 = torch.cat([F.scaled_dot_product_attention(q2, k2, h) for h in halves], dim=-1)
+    stream1 = torch.cat([F.scaled_dot_product_attention(q1, k1, h, is_causal=causal) for h in halves], dim=-1)
+    stream2 = torch.cat([F.scaled_dot_product_attention(q2, k2, h, is_causal=causal) for h in halves], dim=-1)
     out = stream1 - lambda_scale * stream2
     if rms_norm:
         out = (1 - lambda_init) * _rms(out)

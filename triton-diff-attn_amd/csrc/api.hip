@@ -38,7 +38,7 @@ WsLayout ws_layout(int BH, int N, int D) {
 
 extern "C" {
 
-int diffattn_abi_version(void) { return 1; }
+int diffattn_abi_version(void) { return 2; }
 
 const char* diffattn_strerror(int code) {
   switch (code) {
@@ -48,6 +48,7 @@ const char* diffattn_strerror(int code) {
     case DIFFATTN_EINVAL_SEQ: return "N must be a multiple of 128";
     case DIFFATTN_EINVAL_WS: return "workspace too small or misaligned";
     case DIFFATTN_EINVAL_ALIGN: return "tensor pointers must be 16-byte aligned";
+    case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL)";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -56,9 +57,10 @@ const char* diffattn_strerror(int code) {
 
 int diffattn_forward(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
                      const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
-                     int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                     int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                      void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y) return DIFFATTN_EINVAL_NULL;
+  if (flags & ~(DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL)) return DIFFATTN_EINVAL_FLAGS;
   if (int e = check_dims(B, H, N, D)) return e;
   if (!aligned16(q1) || !aligned16(q2) || !aligned16(k1) || !aligned16(k2) || !aligned16(v) ||
       !aligned16(y) || !aligned16(u2))
@@ -67,7 +69,7 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
   p.q1 = (const half_t*)q1; p.q2 = (const half_t*)q2; p.k1 = (const half_t*)k1; p.k2 = (const half_t*)k2;
   p.v = (const half_t*)v; p.lambda_scale = (const half_t*)lambda_scale;
   p.y = (half_t*)y; p.u2 = (half_t*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
-  p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = rms_norm ? 1 : 0;
+  p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0; p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
   return (int)launch_fwd(p, D, (hipStream_t)stream);
 }
 
@@ -81,12 +83,13 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              const float* lse1, const float* lse2, const float* rinv, const void* dy,
                              void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                              void* workspace, size_t workspace_bytes,
-                             int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                             int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                              unsigned stage_mask, void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy ||
       !dq1 || !dq2 || !dk1 || !dk2 || !dv || !dlambda || !workspace)
     return DIFFATTN_EINVAL_NULL;
-  if (rms_norm && !rinv) return DIFFATTN_EINVAL_NULL;
+  if (flags & ~(DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL)) return DIFFATTN_EINVAL_FLAGS;
+  if ((flags & DIFFATTN_RMS_NORM) && !rinv) return DIFFATTN_EINVAL_NULL;
   if (int e = check_dims(B, H, N, D)) return e;
   const void* ptrs[] = {q1, q2, k1, k2, v, y, u2, dy, dq1, dq2, dk1, dk2, dv};
   for (const void* q : ptrs)
@@ -103,7 +106,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   p.dlambda = (half_t*)dlambda;
   p.dx = (half_t*)(ws + w.dx); p.stat = (float*)(ws + w.stat);
   p.dlam_part = (float*)(ws + w.part); p.n_part = bwd_num_partials(B * H, N, D);
-  p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = rms_norm ? 1 : 0;
+  p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0; p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
   p.stages = stage_mask & DIFFATTN_STAGE_ALL;
   return (int)launch_bwd(p, D, (hipStream_t)stream);
 }
@@ -113,11 +116,11 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
                       const float* lse1, const float* lse2, const float* rinv, const void* dy,
                       void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                       void* workspace, size_t workspace_bytes,
-                      int B, int H, int N, int D, float sm_scale, float lambda_init, int rms_norm,
+                      int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                       void* stream) {
   return diffattn_backward_stages(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy,
                                   dq1, dq2, dk1, dk2, dv, dlambda, workspace, workspace_bytes,
-                                  B, H, N, D, sm_scale, lambda_init, rms_norm, DIFFATTN_STAGE_ALL, stream);
+                                  B, H, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, stream);
 }
 
 }  // extern "C"

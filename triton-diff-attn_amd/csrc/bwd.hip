@@ -135,7 +135,8 @@ struct DkvCfg {
 // MODE 0 computes dV, dK1 and dK2 in one pass.  At D = 128 their accumulators plus the resident
 // K1, K2, V rows exceed the 512 registers of a lane, so the work is split in two launches:
 // MODE 1 computes dV only (scores S1, S2; no dP), MODE 2 computes dK1 and dK2 only.
-template <int D, int MODE>
+// CAUSAL: queries before the key block are skipped and the four sub-tiles on the diagonal are masked.
+template <int D, int MODE, bool CAUSAL>
 __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_kernel(BwdParams p) {
   using C = DkvCfg<D>;
   constexpr int DV = C::DV, NW = C::NW, BK = C::BK, BQ = C::BQ;
@@ -287,9 +288,14 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   // stages that are issued one product apart, so that no VALU instruction waits on the one
   // before it: (1) exponentials, (2) products, (3) fp16 packing of a pair of rows.
   struct RowTmp { float p1[16], p2[16], u[16], ds1[16], ds2[16], pc[16]; };
-  auto ew1 = [&](int r, const f4v& st3, const Scores& in, RowTmp& t) {
+  // `rel` (masked steps only) = key index minus the query index of register 0 of the sub-tile:
+  // register r holds query 8*(r/4) + (r%4) relative to that, and a query before its key sees nothing
+  auto ew1 = [&](int r, const f4v& st3, const Scores& in, RowTmp& t, auto masked_tag, int rel) {
     t.p1[r] = fast_exp2(in.s1[r]);
     t.p2[r] = fast_exp2(in.s2[r]);
+    if constexpr (decltype(masked_tag)::value) {
+      if (8 * (r / 4) + (r % 4) < rel) { t.p1[r] = 0.f; t.p2[r] = 0.f; }
+    }
     if constexpr (DO_K) {
       t.u[r] = __builtin_fmaf(-lam, in.dp[r], st3[r % 4]);
       asm volatile("" : "+v"(t.p1[r]), "+v"(t.p2[r]), "+v"(t.u[r]));   // computed here, not moved to its use
@@ -315,8 +321,8 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     }
   };
   // slot s of the skewed schedule: stage 1 of row s, stage 2 of row s-1, stage 3 of the pair ending at row s-2
-  auto ew_slot = [&](int s, const f4v (&st)[4], const Scores& in, RowTmp& t, Packed& out) {
-    if (s < 16) ew1(s, st[s / 4], in, t);
+  auto ew_slot = [&](int s, const f4v (&st)[4], const Scores& in, RowTmp& t, Packed& out, auto masked_tag, int rel) {
+    if (s < 16) ew1(s, st[s / 4], in, t, masked_tag, rel);
     if (s >= 1 && s - 1 < 16) ew2(s - 1, in, t);
     if (s >= 2 && s - 2 < 16 && ((s - 2) & 1)) ew3(s - 2, t, out);
   };
@@ -352,6 +358,9 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   const int n_qt = p.N / BQ;
   const int n_sub = p.N / 32;
   auto buf_of = [](int tile) { return tile % C::NBUF; };
+  // first sub-tile and tile of the loop: with the causal mask no query before the key block matters
+  const int i0 = CAUSAL ? kt * (BK / 32) : 0;
+  const int t0 = i0 / SPT;
 
   // One step.  Chunk k holds score product k of sub-tile (bufn, qsn), every RATIO-th chunk also
   // accumulate product (k/RATIO + NACC/2) % NACC -- the upper query half of sub-tile (bufp, qsp)
@@ -362,7 +371,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   static_assert(NPROD % 16 == 0 || 16 % NPROD == 0, "rows are spread evenly over the products");
   constexpr int AHEAD = 3;                     // B fragments requested ahead of their product
   auto fused = [&](int bufn, int qsn, Scores& s_nxt, int bufc, int qsc, const Scores& s_cur, Packed& pk,
-                   int bufp, int qsp, int tile_next, int buf_next, bool fetch) {
+                   int bufp, int qsp, int tile_next, int buf_next, bool fetch, auto masked_tag, int rel) {
     constexpr int NSLOT = 18;                  // 16 rows + 2 slots of pipeline drain
     constexpr int LEAD = 2;                    // slots run before the first product
     // rows 0..7 are packed by slot 9, which must precede the first product that reads them
@@ -382,7 +391,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     for (int k = 0; k < AHEAD; ++k) bf[k] = bfrag(k);
     // the first slots run while the initial accumulator values and the first fragments arrive
 #pragma unroll
-    for (int s = 0; s < LEAD; ++s) ew_slot(s, st, s_cur, tmp, pk);
+    for (int s = 0; s < LEAD; ++s) ew_slot(s, st, s_cur, tmp, pk, masked_tag, rel);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int k = 0; k < NPROD; ++k) {
@@ -397,7 +406,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
       // slots LEAD .. NSLOT-1 spread over the products
       const int s0 = LEAD + (NSLOT - LEAD) * k / NPROD, s1 = LEAD + (NSLOT - LEAD) * (k + 1) / NPROD;
 #pragma unroll
-      for (int s = s0; s < s1; ++s) ew_slot(s, st, s_cur, tmp, pk);
+      for (int s = s0; s < s1; ++s) ew_slot(s, st, s_cur, tmp, pk, masked_tag, rel);
       __builtin_amdgcn_sched_barrier(0);
     }
     // the next step's VALU reads these results right away
@@ -405,12 +414,12 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   };
 
   // step i: compile-time positions of sub-tiles i+1, i, i-1 inside their tiles
-  auto step = [&](int i, auto subn_tag, const Scores& s_cur, Scores& s_nxt, Packed& pk) {
+  auto step = [&](int i, auto subn_tag, const Scores& s_cur, Scores& s_nxt, Packed& pk, auto masked_tag) {
     constexpr int SUBN = decltype(subn_tag)::value;           // (i + 1) % SPT
     constexpr int SUBC = (SUBN + SPT - 1) % SPT;              // i % SPT
     constexpr int SUBP = (SUBN + 2 * SPT - 2) % SPT;          // (i - 1) % SPT
     const bool more = (i + 1 < n_sub);
-    const int tn = (more ? i + 1 : i) / SPT, tc = i / SPT, tp = (i > 0 ? i - 1 : 0) / SPT;
+    const int tn = (more ? i + 1 : i) / SPT, tc = i / SPT, tp = (i > i0 ? i - 1 : i0) / SPT;
     const bool opens = (SUBN == 0 && more);
     if (opens) {
       // sub-tile i+1 opens tile tn: its data must have landed; tile tn+1 is fetched during this step
@@ -419,18 +428,21 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     }
     const int tl = (tn + 1 < n_qt) ? tn + 1 : tn;             // past the end: harmless re-read
     // past the end the last sub-tile is scored again and the result is never used; before the
-    // start the all-zero upper operand half is accumulated against tile 0
+    // start the all-zero upper operand half is accumulated against the first tile
     fused(buf_of(tn), more ? SUBN : SUBC, s_nxt, buf_of(tc), SUBC, s_cur, pk,
-          buf_of(tp), (i > 0) ? SUBP : 0, tl, buf_of(tn + 1), opens);
+          buf_of(tp), (i > i0) ? SUBP : 0, tl, buf_of(tn + 1), opens, masked_tag, key - 32 * i - 4 * g);
   };
 
-  // prologue: tile 0, then start fetching tile 1; scores of sub-tile 0
-  stage(0, 0, 0); stage(0, 0, 1); stage(0, 0, 2); stage(0, 0, 3);
+  // prologue: the first tile, then start fetching the second; scores of the first sub-tile
+  {
+    const int b0 = buf_of(t0);
+    stage(t0, b0, 0); stage(t0, b0, 1); stage(t0, b0, 2); stage(t0, b0, 3);
+  }
   wait_async_tiles();
   __syncthreads();
   {
-    const int t1 = (n_qt > 1) ? 1 : 0;
-    stage(t1, 1, 0); stage(t1, 1, 1); stage(t1, 1, 2); stage(t1, 1, 3);
+    const int t1 = (t0 + 1 < n_qt) ? t0 + 1 : t0, b1 = buf_of(t0 + 1);
+    stage(t1, b1, 0); stage(t1, b1, 1); stage(t1, b1, 2); stage(t1, b1, 3);
   }
   Scores sa, sb;
   Packed pk;
@@ -438,14 +450,26 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
     for (int e = 0; e < 8; ++e) { pk.pc[kk][e] = (half_t)0.f; pk.d1[kk][e] = (half_t)0.f; pk.d2[kk][e] = (half_t)0.f; }
-  init_scores(0, 0, sa);
+  init_scores(buf_of(t0), 0, sa);
 #pragma unroll
-  for (int k = 0; k < NPROD; ++k) prod_mfma(k, prod_frag(0, 0, k), sa);
+  for (int k = 0; k < NPROD; ++k) prod_mfma(k, prod_frag(buf_of(t0), 0, k), sa);
   results_ready(sa);
 
-  for (int i = 0; i < n_sub; i += 2) {   // the sub-tile count is even
-    step(i, std::integral_constant<int, 1 % SPT>{}, sa, sb, pk);
-    step(i + 1, std::integral_constant<int, 2 % SPT>{}, sb, sa, pk);
+  constexpr std::integral_constant<int, 1 % SPT> even_tag{};   // position of sub-tile i+1 in its tile, i even
+  constexpr std::integral_constant<int, 2 % SPT> odd_tag{};
+  int i = i0;
+  if constexpr (CAUSAL) {
+    // the key block's own four sub-tiles straddle the diagonal: wave w masks sub-tiles i0 .. i0+w
+    static_assert(BK == 128, "four diagonal sub-tiles per key block");
+    step(i0, even_tag, sa, sb, pk, std::true_type{});
+    step(i0 + 1, odd_tag, sb, sa, pk, std::true_type{});
+    step(i0 + 2, even_tag, sa, sb, pk, std::true_type{});
+    step(i0 + 3, odd_tag, sb, sa, pk, std::true_type{});
+    i = i0 + 4;
+  }
+  for (; i < n_sub; i += 2) {   // an even number of sub-tiles remains
+    step(i, even_tag, sa, sb, pk, std::false_type{});
+    step(i + 1, odd_tag, sb, sa, pk, std::false_type{});
   }
   // upper query half of the last sub-tile
 #pragma unroll
@@ -494,7 +518,7 @@ struct DqCfg {
 // dQ_t = s * dS_t K_t for one block of query rows.  Every product is formed transposed,
 // [keys x queries], so that a lane owns one query column: the row statistics are per-lane
 // scalars and dS^T in accumulator layout is directly the B operand of dQ^T = K^T dS^T.
-template <int D, int NWAVES>
+template <int D, int NWAVES, bool CAUSAL>
 __global__ __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(DqCfg<D, NWAVES>::OCC, DqCfg<D, NWAVES>::OCC))) void bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<D, NWAVES>;
   constexpr int DV = C::DV, NW = C::NW, BM = C::BM, BN = C::BN;
@@ -508,7 +532,8 @@ __global__ __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(DqC
 
   const int n_qt = p.N / BM;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = tile / n_qt, qt = tile % n_qt;
+  // causal: the query blocks of a (batch, head) are visited last to first, longest loops first
+  const int bh = tile / n_qt, qt = CAUSAL ? (n_qt - 1 - tile % n_qt) : (tile % n_qt);
   const size_t rows = (size_t)p.BH * p.N;
   const size_t row0 = (size_t)bh * p.N;
   const size_t qrow = row0 + qt * BM + wave * 32 + j;
@@ -549,7 +574,8 @@ __global__ __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(DqC
   const half_t* gk1 = p.k1 + row0 * D;
   const half_t* gk2 = p.k2 + row0 * D;
   const half_t* gv = p.v + row0 * DV;
-  const int n_tiles = p.N / BN;
+  // causal: keys beyond the last row of the workgroup are never visited
+  const int n_tiles = CAUSAL ? (qt + 1) * (BM / BN) : p.N / BN;
   constexpr int VH = (VTile::PER + 1) / 2;
 
   const int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
@@ -597,6 +623,17 @@ __global__ __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(DqC
       }
       if (ksub == 0) VTile::template issue<0, VH>(gv + (size_t)tn * BN * DV, nb + 2 * C::K_TILE, wave, lane);
       if (ksub == BN / 32 - 1) VTile::template issue<VH, VTile::PER>(gv + (size_t)tn * BN * DV, nb + 2 * C::K_TILE, wave, lane);
+      if constexpr (CAUSAL) {
+        // only the last sub-tiles of a wave's loop reach past its first row: mask key > query there
+        const int wrow0 = qt * BM + wave * 32;
+        const int kbase = t * BN + ksub * 32;
+        if (kbase + 31 > wrow0) {
+          const int rel = wrow0 + j - kbase - 4 * g;     // query index minus the key index of register 0
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (8 * (r / 4) + (r % 4) > rel) { s1[r] = -INFINITY; s2[r] = -INFINITY; }
+        }
+      }
       h8 b1[2], b2[2];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -668,21 +705,27 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
   if (p.stages & 4u) {
     const dim3 grid(p.BH * (p.N / DkvCfg<D>::BK)), block(DkvCfg<D>::NT);
     if constexpr (D == 128) {
-      hipLaunchKernelGGL((bwd_dkdv_kernel<D, 1>), grid, block, 0, stream, p);
+      if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, 1, true>), grid, block, 0, stream, p);
+      else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, 1, false>), grid, block, 0, stream, p);
       if ((e = hipGetLastError()) != hipSuccess) return e;
-      hipLaunchKernelGGL((bwd_dkdv_kernel<D, 2>), grid, block, 0, stream, p);
+      if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, 2, true>), grid, block, 0, stream, p);
+      else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, 2, false>), grid, block, 0, stream, p);
     } else {
-      hipLaunchKernelGGL((bwd_dkdv_kernel<D, 0>), grid, block, 0, stream, p);
+      if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, 0, true>), grid, block, 0, stream, p);
+      else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, 0, false>), grid, block, 0, stream, p);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 8u) {
     // 256 query rows per workgroup when the sequence allows it, otherwise 128; a D = 128 workgroup
     // runs one wave per SIMD and therefore has four waves
-    if (p.N % 256 == 0 && D != 128)
-      hipLaunchKernelGGL((bwd_dq_kernel<D, 8>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
-    else
-      hipLaunchKernelGGL((bwd_dq_kernel<D, 4>), dim3(p.BH * (p.N / 128)), dim3(256), 0, stream, p);
+    if (p.N % 256 == 0 && D != 128) {
+      if (p.causal) hipLaunchKernelGGL((bwd_dq_kernel<D, 8, true>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
+      else          hipLaunchKernelGGL((bwd_dq_kernel<D, 8, false>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
+    } else {
+      if (p.causal) hipLaunchKernelGGL((bwd_dq_kernel<D, 4, true>), dim3(p.BH * (p.N / 128)), dim3(256), 0, stream, p);
+      else          hipLaunchKernelGGL((bwd_dq_kernel<D, 4, false>), dim3(p.BH * (p.N / 128)), dim3(256), 0, stream, p);
+    }
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   return e;

@@ -38,7 +38,7 @@ struct FwdCfg {
 
 constexpr float kRescaleThreshold = 8.0f;   // log2 units: probabilities stay below 2^8 between updates of the row max
 
-template <int D, bool RMS>
+template <int D, bool RMS, bool CAUSAL>
 __global__ __launch_bounds__(FwdCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::OCC, FwdCfg<D>::OCC)))
 void fwd_kernel(FwdParams p) {
   using C = FwdCfg<D>;
@@ -59,7 +59,8 @@ void fwd_kernel(FwdParams p) {
 
   const int n_qt = p.N / BM;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = tile / n_qt, qt = tile % n_qt;
+  // causal: the query blocks of a (batch, head) are visited last to first, longest loops first
+  const int bh = tile / n_qt, qt = CAUSAL ? (n_qt - 1 - tile % n_qt) : (tile % n_qt);
   const size_t qk_base = (size_t)bh * p.N * D;
   const size_t v_base = (size_t)bh * p.N * DV;
   const int qrow0 = qt * BM + qw * 32 * QS + j;   // this lane's query row of block qs is qrow0 + 32*qs
@@ -105,7 +106,10 @@ void fwd_kernel(FwdParams p) {
   const half_t* gk1 = p.k1 + qk_base;
   const half_t* gk2 = p.k2 + qk_base;
   const half_t* gv = p.v + v_base;
-  const int n_tiles = p.N / BN;
+  // causal: keys beyond the last row of the workgroup are never visited (BM is a multiple of 2*BN,
+  // so the tile count stays even)
+  const int n_tiles = CAUSAL ? (qt + 1) * (BM / BN) : p.N / BN;
+  static_assert(BM % (2 * BN) == 0, "an even number of key tiles per query block");
   constexpr int VH = (VTile::PER + 1) / 2;   // V instructions are issued in two groups
   auto load_k1 = [&](int tk, int buf) { KTile::issue(gk1 + (size_t)tk * BN * D, sKbuf + buf * C::K_BUF, wave, lane); };
   auto load_k2 = [&](int tk, int buf) { KTile::issue(gk2 + (size_t)tk * BN * D, sKbuf + buf * C::K_BUF + C::K_TILE, wave, lane); };
@@ -171,6 +175,20 @@ void fwd_kernel(FwdParams p) {
     // while they arrive.
     h8 ka[NKT][NKS];
     read_k(sKbuf + kb1 * C::K_BUF + st * C::K_TILE, ka);
+
+    if constexpr (CAUSAL) {
+      // only the last tiles of a wave's loop reach past its first row: mask key > query there
+      static_assert(QS == 1, "one 32-row block per wave");
+      const int wrow0 = qt * BM + qw * 32;
+      if ((t + 1) * BN - 1 > wrow0) {
+        const int rel = wrow0 + j - t * BN - 4 * g;      // query index minus the key index of register 0, tile 0
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (kt * 32 + 8 * (r / 4) + (r % 4) > rel) s_cur[0][kt][r] = -INFINITY;
+      }
+    }
 
     float mx[QS];
 #pragma unroll
@@ -340,13 +358,21 @@ void fwd_kernel(FwdParams p) {
   }
 }
 
+template <int D, bool RMS>
+static void launch_fwd_c(const FwdParams& p, dim3 grid, dim3 block, hipStream_t stream) {
+  if (p.causal)
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, true>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, false>), grid, block, 0, stream, p);
+}
+
 template <int D>
 static hipError_t launch_fwd_t(const FwdParams& p, hipStream_t stream) {
   dim3 grid(p.BH * (p.N / FwdCfg<D>::BM)), block(FwdCfg<D>::NT);
   if (p.rms_norm)
-    hipLaunchKernelGGL((fwd_kernel<D, true>), grid, block, 0, stream, p);
+    launch_fwd_c<D, true>(p, grid, block, stream);
   else
-    hipLaunchKernelGGL((fwd_kernel<D, false>), grid, block, 0, stream, p);
+    launch_fwd_c<D, false>(p, grid, block, stream);
   return hipGetLastError();
 }
 

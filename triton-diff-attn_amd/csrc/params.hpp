@@ -15,6 +15,7 @@ struct FwdParams {
   int BH, N;
   float sm_scale, lambda_init;
   int rms_norm;
+  int causal;                   // query i sees keys 0..i only
 };
 
 struct BwdParams {
@@ -33,6 +34,7 @@ struct BwdParams {
   int BH, N;
   float sm_scale, lambda_init;
   int rms_norm;
+  int causal;
   unsigned stages;              // bit 0 row preprocess, 1 d(lambda) reduce, 2 dK/dV, 3 dQ
 };
 

@@ -1,7 +1,8 @@
 """Autograd wiring of the MI355X differential-attention kernels.
 
 Host-side counterpart of the reference's `_diff_attention` (src/kernel.py:461-575): same class
-name, same `apply` argument order, same 9-slot gradient tuple.  The work itself is done by the
+name, same `apply` argument order, same 9-slot gradient tuple (a tenth, optional argument `causal`
+-- masking is a feature the reference lists as missing, src/kernel.py:4 -- adds a tenth slot).  The work itself is done by the
 hand-written HIP kernels in libdiffattn.so, reached through its C ABI; if the library is missing
 the call raises -- there is no other path.
 """
@@ -11,6 +12,8 @@ import _native
 
 _SUPPORTED_D = (32, 64, 128)
 _SEQ_MULTIPLE = 128
+_FLAG_RMS_NORM = 1      # DIFFATTN_RMS_NORM
+_FLAG_CAUSAL = 2        # DIFFATTN_CAUSAL
 
 
 def _check_inputs(Q1, Q2, K1, K2, V):
@@ -57,13 +60,14 @@ def _ptr(t):
 class _diff_attention(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, Q1, Q2, K1, K2, V, SM_SCALE, LAMBDA_SCALE, LAMBDA_INIT, rms_norm=False):
+    def forward(ctx, Q1, Q2, K1, K2, V, SM_SCALE, LAMBDA_SCALE, LAMBDA_INIT, rms_norm=False, causal=False):
         B, H, N, D = _check_inputs(Q1, Q2, K1, K2, V)
         lib = _native.lib()
         dev = Q1.device
         q1, q2, k1, k2, v = (t.contiguous() for t in (Q1, Q2, K1, K2, V))
         lam = _lambda_tensor(LAMBDA_SCALE, dev)
         rms_norm = bool(rms_norm)
+        flags = (_FLAG_RMS_NORM if rms_norm else 0) | (_FLAG_CAUSAL if causal else 0)
 
         y = torch.empty_like(v)
         u2 = torch.empty_like(v)
@@ -76,12 +80,12 @@ class _diff_attention(torch.autograd.Function):
             _native.check(lib.diffattn_forward(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
                 lam.data_ptr(), y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv),
-                B, H, N, D, float(SM_SCALE), float(LAMBDA_INIT), int(rms_norm), stream))
+                B, H, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, stream))
 
         ctx.save_for_backward(q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam)
         ctx.SM_SCALE = float(SM_SCALE)
         ctx.LAMBDA_INIT = float(LAMBDA_INIT)
-        ctx.RMS_NORM = rms_norm
+        ctx.FLAGS = flags
         ctx.lambda_meta = (LAMBDA_SCALE.dtype, LAMBDA_SCALE.shape) if torch.is_tensor(LAMBDA_SCALE) else None
         return y
 
@@ -108,10 +112,11 @@ class _diff_attention(torch.autograd.Function):
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv), dO.data_ptr(),
                 dq1.data_ptr(), dq2.data_ptr(), dk1.data_ptr(), dk2.data_ptr(), dv.data_ptr(), dlam.data_ptr(),
-                ws.data_ptr(), ws_bytes, B, H, N, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, int(ctx.RMS_NORM), stream))
+                ws.data_ptr(), ws_bytes, B, H, N, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stream))
 
         dlambda = None
         if ctx.lambda_meta is not None and ctx.needs_input_grad[6]:
             dtype, shape = ctx.lambda_meta
             dlambda = dlam.to(dtype).reshape(shape)
-        return dq1, dq2, dk1, dk2, dv, None, dlambda, None, None
+        # one slot per forward argument: nine, or ten when `causal` was passed
+        return (dq1, dq2, dk1, dk2, dv, None, dlambda) + (None,) * (len(ctx.needs_input_grad) - 7)

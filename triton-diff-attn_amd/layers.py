@@ -18,14 +18,18 @@ def MultiheadDiffAttnKernel(
     lambda_scale=-0.5,
     lambda_init: float = 0.8,
     rms_norm: bool = False,
+    causal: bool = False,
 ):
     """(softmax(q1 k1^T / sqrt(d)) - lambda_scale * softmax(q2 k2^T / sqrt(d))) v, optionally followed
     by a per-row RMSNorm over the 2d output features and a (1 - lambda_init) scale.
 
     q1, q2, k1, k2: [B, H, N, d] fp16 on the GPU; v: [B, H, N, 2d]; lambda_scale: 1-element tensor
     (a python float is accepted too).  Returns [B, H, N, 2d] fp16 with autograd support for the
-    five tensors and lambda_scale.
+    five tensors and lambda_scale.  `causal` (not in the reference, which lists masking as missing,
+    src/kernel.py:4) lets query i attend to keys 0..i only.
     """
     head_dim = q1.size(-1)
     sm_scale = 1 / math.sqrt(head_dim)
+    if causal:
+        return _diff_attention.apply(q1, q2, k1, k2, v, sm_scale, lambda_scale, lambda_init, rms_norm, True)
     return _diff_attention.apply(q1, q2, k1, k2, v, sm_scale, lambda_scale, lambda_init, rms_norm)

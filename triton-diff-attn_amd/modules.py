@@ -4,7 +4,7 @@ The reference stops at the functional operator (src/layers.py:10-26); its kernel
 the Differential Transformer paper (src/kernel.py:1) for the layer around it.  This module is that
 layer: input projections, the re-parametrised lambda, the fused operator with its per-head RMSNorm
 and (1 - lambda_init) scale, a learnable per-feature gain on the normalised heads, and the output
-projection.  Attention is bidirectional, like the operator.
+projection.  Attention is bidirectional unless `causal=True`.
 
   x [B, N, E]  ->  q, k [B, 2H, N, d],  v [B, H, N, 2d]      (E = 2 * H * d)
   lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + lambda_init       (one scalar per layer)
@@ -26,7 +26,7 @@ def lambda_init_for_depth(depth: int) -> float:
 
 class DiffAttn(nn.Module):
     def __init__(self, embed_dim: int, num_heads: int, depth: int = 0, attention=MultiheadDiffAttnKernel,
-                 device=None, dtype=torch.float16):
+                 causal: bool = False, device=None, dtype=torch.float16):
         super().__init__()
         if embed_dim % (2 * num_heads) != 0:
             raise ValueError("embed_dim must be divisible by 2 * num_heads")
@@ -35,6 +35,7 @@ class DiffAttn(nn.Module):
         self.head_dim = embed_dim // (2 * num_heads)      # d: q/k sub-head width; a value head is 2d wide
         self.lambda_init = lambda_init_for_depth(depth)
         self.attention = attention
+        self.causal = causal
         kw = dict(device=device, dtype=dtype)
         self.q_proj = nn.Linear(embed_dim, embed_dim, bias=False, **kw)
         self.k_proj = nn.Linear(embed_dim, embed_dim, bias=False, **kw)
@@ -62,6 +63,7 @@ class DiffAttn(nn.Module):
         v = self.v_proj(x).view(B, N, H, 2 * d).transpose(1, 2)
         lam = self.lambda_scale().to(x.dtype)
         heads = self.attention(q[0].contiguous(), q[1].contiguous(), k[0].contiguous(), k[1].contiguous(),
-                               v.contiguous(), lambda_scale=lam, lambda_init=self.lambda_init, rms_norm=True)
+                               v.contiguous(), lambda_scale=lam, lambda_init=self.lambda_init, rms_norm=True,
+                               **({"causal": True} if self.causal else {}))
         heads = heads * self.head_gain
         return self.out_proj(heads.transpose(1, 2).reshape(B, N, E))
