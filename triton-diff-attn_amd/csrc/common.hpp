@@ -38,11 +38,6 @@ __device__ __forceinline__ f16v mfma32(h8 a, h8 b, f16v c) {
 // file for the whole kernel, at no cost in VGPRs and without copies.  Being inline assembly, the
 // compiler does not know these are matrix instructions: the caller must put mfma_results_ready()
 // between the last of them and the first VALU read of the result.
-__device__ __forceinline__ f16v mfma32_bagpr_first(h8 a, h8 b) {
-  f16v d;
-  asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
-  return d;
-}
 __device__ __forceinline__ f16v mfma32_bagpr(h8 a, h8 b, f16v c) {
   asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
   return c;
@@ -189,34 +184,6 @@ __device__ __forceinline__ void wait_async_tiles_except(int newest) {
     default: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
   }
 }
-
-// Cooperative copy of a dense [ROWS x COLS] fp16 tile (row stride COLS in global memory) into an
-// LDS tile with row stride STRIDE, staged through registers so the global loads of the next tile
-// can be in flight while the current one is consumed.
-template <int ROWS, int COLS, int STRIDE, int NT>
-struct TileStage {
-  static constexpr int CPR = COLS / 8;           // 16-byte chunks per row
-  static constexpr int NCH = ROWS * CPR;
-  static constexpr int PER = (NCH + NT - 1) / NT;
-  u32x4 reg[PER];
-  __device__ __forceinline__ void load(const half_t* __restrict__ g, int tid) {
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      int c = tid + i * NT;
-      if (NCH % NT == 0 || c < NCH) reg[i] = *reinterpret_cast<const u32x4*>(g + (size_t)c * 8);
-    }
-  }
-  __device__ __forceinline__ void store(half_t* s, int tid) const {
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      int c = tid + i * NT;
-      if (NCH % NT == 0 || c < NCH) {
-        int row = c / CPR, col = c % CPR;
-        *reinterpret_cast<u32x4*>(s + row * STRIDE + col * 8) = reg[i];
-      }
-    }
-  }
-};
 
 // Workgroup id -> logical tile id such that consecutive logical ids land on the same XCD
 // (workgroups are dealt round-robin to the 8 XCDs, each with a private L2).
