@@ -30,7 +30,7 @@ extern "C" {
 #define DIFFATTN_OK 0
 #define DIFFATTN_EINVAL_NULL (-1)   /* a required pointer is null */
 #define DIFFATTN_EINVAL_DIM (-2)    /* D not in {32,64,128} or B,H,N not positive */
-#define DIFFATTN_EINVAL_SEQ (-3)    /* N not a multiple of 128 */
+#define DIFFATTN_EINVAL_SEQ (-3)    /* N not a multiple of 128, or n_valid outside 1..N */
 #define DIFFATTN_EINVAL_WS (-4)     /* workspace too small */
 #define DIFFATTN_EINVAL_ALIGN (-5)  /* a pointer is not 16-byte aligned */
 #define DIFFATTN_EINVAL_FLAGS (-6)  /* unknown bits in `flags` */
@@ -64,6 +64,19 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
                      const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
                      int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                      void* stream);
+
+/*
+ * Forward for a sequence whose real length n_valid is not a multiple of 128.  No counterpart in the
+ * reference, whose kernels require such a multiple (src/kernel.py:4, :527).  The caller pads every
+ * tensor with zero rows to N (a multiple of 128, n_valid <= N); keys n_valid..N-1 are ignored, rows
+ * n_valid..N-1 of the outputs are to be discarded.  The backward needs no variant: with zero rows of
+ * k1, k2, v and dy in the padding, diffattn_backward on the padded tensors returns the exact
+ * gradients in rows 0..n_valid-1.  diffattn_forward is this function with n_valid = N.
+ */
+int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                            const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
+                            int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
+                            void* stream);
 
 /* Bytes of device workspace diffattn_backward needs for this problem size (0 on bad sizes). */
 size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D);

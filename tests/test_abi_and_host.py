@@ -19,7 +19,7 @@ def declared_symbols():
 
 def test_header_declares_the_expected_entry_points():
     assert declared_symbols() == sorted([
-        "diffattn_abi_version", "diffattn_strerror", "diffattn_forward",
+        "diffattn_abi_version", "diffattn_strerror", "diffattn_forward", "diffattn_forward_padded",
         "diffattn_backward_workspace_bytes", "diffattn_backward", "diffattn_backward_stages"])
 
 
@@ -49,6 +49,9 @@ def test_argument_rejection_needs_no_gpu():
     bad = args(1, 1, 128, 64)
     bad[-2] = 4                                   # unknown flag bit
     assert lib.diffattn_forward(*bad) == -6
+    padded = lambda n_valid: [p] * 11 + [1, 1, 128, n_valid, 64, 0.125, 0.8, 1, None]
+    assert lib.diffattn_forward_padded(*padded(0)) == -3
+    assert lib.diffattn_forward_padded(*padded(129)) == -3
     assert lib.diffattn_backward_workspace_bytes(1, 1, 100, 64) == 0
     assert lib.diffattn_backward_workspace_bytes(1, 1, 128, 48) == 0
     need = lib.diffattn_backward_workspace_bytes(2, 3, 256, 64)
@@ -77,6 +80,12 @@ def test_host_validation_errors():
         _check_inputs(*[t(1, 1, 128, 64)] * 4, t(1, 1, 128, 128))
     with pytest.raises(ValueError):
         _lambda_tensor(torch.zeros(2), torch.device("cpu"))
+    from kernel import _pad_rows
+    x = torch.arange(2 * 3 * 5 * 4, dtype=torch.float16).reshape(2, 3, 5, 4)
+    padded = _pad_rows(x, 8)
+    assert padded.shape == (2, 3, 8, 4) and padded.is_contiguous()
+    assert torch.equal(padded[:, :, :5], x) and padded[:, :, 5:].abs().sum() == 0
+    assert _pad_rows(x, 5) is x
     lam = _lambda_tensor(0.25, torch.device("cpu"))
     assert lam.dtype == torch.float16 and lam.shape == (1,) and lam.item() == 0.25
 

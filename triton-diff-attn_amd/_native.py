@@ -21,6 +21,8 @@ SYMBOLS = {
     "diffattn_strerror": (ctypes.c_char_p, [ctypes.c_int]),
     "diffattn_forward": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp] + [ctypes.c_int] * 4
                          + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
+    "diffattn_forward_padded": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp] + [ctypes.c_int] * 5
+                                + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
     "diffattn_backward_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 4),
     "diffattn_backward": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp, _vp] + [_vp] * 6
                           + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 4

@@ -45,7 +45,7 @@ const char* diffattn_strerror(int code) {
     case DIFFATTN_OK: return "success";
     case DIFFATTN_EINVAL_NULL: return "a required pointer is null";
     case DIFFATTN_EINVAL_DIM: return "unsupported sizes: D must be 32, 64 or 128 and B, H, N positive";
-    case DIFFATTN_EINVAL_SEQ: return "N must be a multiple of 128";
+    case DIFFATTN_EINVAL_SEQ: return "N must be a multiple of 128 (and 1 <= n_valid <= N)";
     case DIFFATTN_EINVAL_WS: return "workspace too small or misaligned";
     case DIFFATTN_EINVAL_ALIGN: return "tensor pointers must be 16-byte aligned";
     case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL)";
@@ -59,9 +59,18 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
                      const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
                      int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                      void* stream) {
+  return diffattn_forward_padded(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv,
+                                 B, H, N, N, D, sm_scale, lambda_init, flags, stream);
+}
+
+int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                            const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
+                            int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
+                            void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y) return DIFFATTN_EINVAL_NULL;
   if (flags & ~(DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL)) return DIFFATTN_EINVAL_FLAGS;
   if (int e = check_dims(B, H, N, D)) return e;
+  if (n_valid < 1 || n_valid > N) return DIFFATTN_EINVAL_SEQ;
   if (!aligned16(q1) || !aligned16(q2) || !aligned16(k1) || !aligned16(k2) || !aligned16(v) ||
       !aligned16(y) || !aligned16(u2))
     return DIFFATTN_EINVAL_ALIGN;
@@ -70,6 +79,7 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
   p.v = (const half_t*)v; p.lambda_scale = (const half_t*)lambda_scale;
   p.y = (half_t*)y; p.u2 = (half_t*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
   p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0; p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
+  p.n_keys = n_valid;
   return (int)launch_fwd(p, D, (hipStream_t)stream);
 }
 

@@ -38,7 +38,9 @@ struct FwdCfg {
 
 constexpr float kRescaleThreshold = 8.0f;   // log2 units: probabilities stay below 2^8 between updates of the row max
 
-template <int D, bool RMS, bool CAUSAL>
+// MASK: 0 none; 1 causal (key <= query); 2 the last keys of the sequence are padding (key < n_keys).
+// With the causal mask the padding needs no extra test: a padded key lies after every real query.
+template <int D, bool RMS, int MASK>
 __global__ __launch_bounds__(FwdCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::OCC, FwdCfg<D>::OCC)))
 void fwd_kernel(FwdParams p) {
   using C = FwdCfg<D>;
@@ -60,6 +62,7 @@ void fwd_kernel(FwdParams p) {
   const int n_qt = p.N / BM;
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
   // causal: the query blocks of a (batch, head) are visited last to first, longest loops first
+  constexpr bool CAUSAL = (MASK == 1), PADDED = (MASK == 2);
   const int bh = tile / n_qt, qt = CAUSAL ? (n_qt - 1 - tile % n_qt) : (tile % n_qt);
   const size_t qk_base = (size_t)bh * p.N * D;
   const size_t v_base = (size_t)bh * p.N * DV;
@@ -182,6 +185,18 @@ void fwd_kernel(FwdParams p) {
       const int wrow0 = qt * BM + qw * 32;
       if ((t + 1) * BN - 1 > wrow0) {
         const int rel = wrow0 + j - t * BN - 4 * g;      // query index minus the key index of register 0, tile 0
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (kt * 32 + 8 * (r / 4) + (r % 4) > rel) s_cur[0][kt][r] = -INFINITY;
+      }
+    }
+
+    if constexpr (PADDED) {
+      // only the last tiles hold padding keys
+      if ((t + 1) * BN > p.n_keys) {
+        const int rel = p.n_keys - 1 - t * BN - 4 * g;   // last real key minus the key index of register 0, tile 0
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
@@ -361,9 +376,11 @@ void fwd_kernel(FwdParams p) {
 template <int D, bool RMS>
 static void launch_fwd_c(const FwdParams& p, dim3 grid, dim3 block, hipStream_t stream) {
   if (p.causal)
-    hipLaunchKernelGGL((fwd_kernel<D, RMS, true>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, 1>), grid, block, 0, stream, p);
+  else if (p.n_keys < p.N)
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, 2>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((fwd_kernel<D, RMS, false>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, 0>), grid, block, 0, stream, p);
 }
 
 template <int D>

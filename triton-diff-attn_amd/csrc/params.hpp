@@ -16,6 +16,7 @@ struct FwdParams {
   float sm_scale, lambda_init;
   int rms_norm;
   int causal;                   // query i sees keys 0..i only
+  int n_keys;                   // keys n_keys..N-1 are padding and are ignored (N when there is none)
 };
 
 struct BwdParams {

@@ -38,9 +38,16 @@ def _check_inputs(Q1, Q2, K1, K2, V):
         raise ValueError("v has shape %s, expected %s" % (tuple(V.shape), (B, H, N, 2 * D)))
     if D not in _SUPPORTED_D:
         raise ValueError("head dim %d unsupported; supported: %s" % (D, _SUPPORTED_D))
-    if N % _SEQ_MULTIPLE != 0:
-        raise ValueError("sequence length %d must be a multiple of %d" % (N, _SEQ_MULTIPLE))
+    if N < 1:
+        raise ValueError("empty sequence")
     return B, H, N, D
+
+
+def _pad_rows(t, n_pad):
+    """[B,H,N,C] -> dense [B,H,n_pad,C] with zero rows appended (the tensor itself when nothing is missing)."""
+    if t.size(2) == n_pad:
+        return t.contiguous()
+    return torch.nn.functional.pad(t, (0, 0, 0, n_pad - t.size(2)))
 
 
 def _lambda_tensor(lambda_scale, device):
@@ -64,30 +71,35 @@ class _diff_attention(torch.autograd.Function):
         B, H, N, D = _check_inputs(Q1, Q2, K1, K2, V)
         lib = _native.lib()
         dev = Q1.device
-        q1, q2, k1, k2, v = (t.contiguous() for t in (Q1, Q2, K1, K2, V))
+        # The kernels work on multiples of 128 rows (like the reference's, src/kernel.py:527).  Other
+        # lengths are padded with zero rows here; the forward ignores the padding keys, and with zero
+        # k, v and upstream-gradient rows there the backward is exact on the real rows.
+        n_pad = -(-N // _SEQ_MULTIPLE) * _SEQ_MULTIPLE
+        q1, q2, k1, k2, v = (_pad_rows(t, n_pad) for t in (Q1, Q2, K1, K2, V))
         lam = _lambda_tensor(LAMBDA_SCALE, dev)
         rms_norm = bool(rms_norm)
         flags = (_FLAG_RMS_NORM if rms_norm else 0) | (_FLAG_CAUSAL if causal else 0)
 
         y = torch.empty_like(v)
         u2 = torch.empty_like(v)
-        lse1 = torch.empty((B, H, N), device=dev, dtype=torch.float32)
-        lse2 = torch.empty((B, H, N), device=dev, dtype=torch.float32)
-        rinv = torch.empty((B, H, N), device=dev, dtype=torch.float32) if rms_norm else None
+        lse1 = torch.empty((B, H, n_pad), device=dev, dtype=torch.float32)
+        lse2 = torch.empty((B, H, n_pad), device=dev, dtype=torch.float32)
+        rinv = torch.empty((B, H, n_pad), device=dev, dtype=torch.float32) if rms_norm else None
 
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream().cuda_stream
-            _native.check(lib.diffattn_forward(
+            _native.check(lib.diffattn_forward_padded(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
                 lam.data_ptr(), y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv),
-                B, H, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, stream))
+                B, H, n_pad, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, stream))
 
         ctx.save_for_backward(q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam)
         ctx.SM_SCALE = float(SM_SCALE)
         ctx.LAMBDA_INIT = float(LAMBDA_INIT)
         ctx.FLAGS = flags
+        ctx.N_VALID = N
         ctx.lambda_meta = (LAMBDA_SCALE.dtype, LAMBDA_SCALE.shape) if torch.is_tensor(LAMBDA_SCALE) else None
-        return y
+        return y if n_pad == N else y[:, :, :N].contiguous()
 
     @staticmethod
     def backward(ctx, dO):
@@ -95,9 +107,10 @@ class _diff_attention(torch.autograd.Function):
         B, H, N, D = q1.shape
         lib = _native.lib()
         dev = q1.device
-        dO = dO.contiguous()
         if dO.dtype != torch.float16:
             dO = dO.to(torch.float16)
+        dO = _pad_rows(dO, N)           # N is the padded length here
+        n_valid = ctx.N_VALID
 
         dq1, dq2 = torch.empty_like(q1), torch.empty_like(q2)
         dk1, dk2 = torch.empty_like(k1), torch.empty_like(k2)
@@ -118,5 +131,7 @@ class _diff_attention(torch.autograd.Function):
         if ctx.lambda_meta is not None and ctx.needs_input_grad[6]:
             dtype, shape = ctx.lambda_meta
             dlambda = dlam.to(dtype).reshape(shape)
+        if n_valid != N:
+            dq1, dq2, dk1, dk2, dv = (t[:, :, :n_valid].contiguous() for t in (dq1, dq2, dk1, dk2, dv))
         # one slot per forward argument: nine, or ten when `causal` was passed
         return (dq1, dq2, dk1, dk2, dv, None, dlambda) + (None,) * (len(ctx.needs_input_grad) - 7)
