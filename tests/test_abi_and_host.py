@@ -42,6 +42,7 @@ def test_argument_rejection_needs_no_gpu():
     assert lib.diffattn_forward(*([None] + args(1, 1, 128, 64)[1:])) == -1
     assert lib.diffattn_forward(*args(1, 1, 128, 48)) == -2
     assert lib.diffattn_forward(*args(0, 1, 128, 64)) == -2
+    assert lib.diffattn_forward(*args(1 << 12, 1 << 10, 128, 64)) == -2      # more than 2^28 rows
     assert lib.diffattn_forward(*args(1, 1, 100, 64)) == -3
     bad = args(1, 1, 128, 64)
     bad[0] = p + 2

@@ -13,6 +13,9 @@ int check_dims(int B, int H, int N, int D) {
   if (B <= 0 || H <= 0 || N <= 0) return DIFFATTN_EINVAL_DIM;
   if (D != 32 && D != 64 && D != 128) return DIFFATTN_EINVAL_DIM;
   if ((long long)B * H > 0x7fffffffLL / 64) return DIFFATTN_EINVAL_DIM;
+  // grid sizes are ints and the statistics copy of the dK/dV kernel uses 32-bit byte offsets
+  // (up to 3*B*H*N floats): keep B*H*N below 2^28 rows (a 68 GiB v tensor at D = 64)
+  if ((long long)B * H * N > (1LL << 28)) return DIFFATTN_EINVAL_DIM;
   if (N % 128 != 0) return DIFFATTN_EINVAL_SEQ;
   return DIFFATTN_OK;
 }
