@@ -1,0 +1,50 @@
+"""Numerical stress on the GPU: large logits (the lazily updated softmax reference must keep up), one-hot
+attention rows, constant inputs, zero upstream gradient.  Same oracle, same tolerances."""
+import pytest
+import torch
+
+from oracle import diff_attn_oracle as orc
+from util import GRAD_RTOL, Y_ATOL, make_inputs, max_abs, rel_to_max, run_kernel
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(q1, q2, k1, k2, v, dy, lam, rms, causal=False, y_atol=Y_ATOL):
+    y, grads = run_kernel(q1, q2, k1, k2, v, lam, 0.8, rms, dy, causal=causal)
+    ref = orc.forward_backward(q1, q2, k1, k2, v, torch.tensor([lam], dtype=torch.float16), dy, 0.8, rms, chunk=1,
+                               causal=causal)
+    assert torch.isfinite(y).all() and all(torch.isfinite(g).all() for g in grads)
+    assert max_abs(y, ref[0]) <= y_atol
+    for name, g, r in zip(("dq1", "dq2", "dk1", "dk2", "dv", "dlambda"), grads, ref[1:]):
+        if r.abs().max().item() < 1e-6:
+            assert g.float().abs().max().item() <= 2e-3, name
+        else:
+            assert rel_to_max(g, r) <= GRAD_RTOL, name
+
+
+@pytest.mark.parametrize("scale,D", [(3.0, 64), (4.0, 32), (2.5, 128)])
+def test_large_logits(scale, D):
+    # scores of order scale^2 * sqrt(D): nearly one-hot softmax rows, row maxima that keep growing along the keys
+    q1, q2, k1, k2, v, dy = make_inputs(1, 2, 512, D, seed=41)
+    q1, q2, k1, k2 = (t * scale for t in (q1, q2, k1, k2))
+    _check(q1.half(), q2.half(), k1.half(), k2.half(), v, dy, 0.5, True)
+
+
+def test_growing_row_maximum():
+    # keys sorted so that every later tile raises the row maximum: the rescale path runs on every tile
+    q1, q2, k1, k2, v, dy = make_inputs(1, 1, 512, 64, seed=42)
+    ramp = torch.linspace(0.2, 3.0, 512).reshape(1, 1, 512, 1)
+    k1 = (k1.abs() * ramp).half(); q1 = q1.abs().half()
+    _check(q1, q2, k1, k2, v, dy, 0.5, True)
+    _check(q1, q2, k1, k2, v, dy, 0.5, False, causal=True)
+
+
+def test_constant_inputs_and_zero_gradient():
+    B, H, N, D = 1, 2, 256, 64
+    one = torch.ones(B, H, N, D, dtype=torch.float16)
+    v = torch.randn(B, H, N, 2 * D, generator=torch.Generator().manual_seed(43)).half()
+    dy = torch.randn(B, H, N, 2 * D, generator=torch.Generator().manual_seed(44)).half()
+    _check(one, one, one, one, v, dy, 0.5, False)            # uniform attention: X = (1 - lambda) mean(V)
+    q1, q2, k1, k2, v, dy = make_inputs(B, H, N, D, seed=45)
+    y, grads = run_kernel(q1, q2, k1, k2, v, 0.5, 0.8, True, torch.zeros_like(dy))
+    assert all(g.abs().max().item() == 0 for g in grads)     # zero upstream gradient gives exactly zero gradients
