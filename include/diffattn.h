@@ -8,7 +8,7 @@
  * operands as plain device pointers and sizes.
  *
  * Conventions (all entry points):
- *   - every tensor is dense row-major fp16 ("half"), [B,H,N,D] for q1,q2,k1,k2 and their
+ *   - every tensor is dense row-major fp16 ("half"; bfloat16 with DIFFATTN_BF16), [B,H,N,D] for q1,q2,k1,k2 and their
  *     gradients, [B,H,N,2D] for v, y, u2, dy, dv; row statistics are fp32 [B,H,N];
  *   - D is 32, 64 or 128; N is a multiple of 128;
  *   - lambda_scale is a DEVICE pointer to one fp16 value (the reference loads it in-kernel,
@@ -42,6 +42,9 @@ extern "C" {
  * one problem must be given the same flags. */
 #define DIFFATTN_RMS_NORM 1
 #define DIFFATTN_CAUSAL 2
+/* Every 16-bit tensor (q1..v, y, u2, dy, the gradients, *lambda_scale, *dlambda) is bfloat16 instead of
+ * fp16.  No counterpart in the reference, whose kernel hard-codes fp16 (src/kernel.py:175-176). */
+#define DIFFATTN_BF16 4
 
 /* ABI version of this header; bumped when a signature changes. */
 int diffattn_abi_version(void);

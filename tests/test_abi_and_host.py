@@ -48,7 +48,7 @@ def test_argument_rejection_needs_no_gpu():
     bad[0] = p + 2
     assert lib.diffattn_forward(*bad) == -5
     bad = args(1, 1, 128, 64)
-    bad[-2] = 4                                   # unknown flag bit
+    bad[-2] = 8                                   # unknown flag bit
     assert lib.diffattn_forward(*bad) == -6
     padded = lambda n_valid: [p] * 11 + [1, 1, 128, n_valid, 64, 0.125, 0.8, 1, None]
     assert lib.diffattn_forward_padded(*padded(0)) == -3
@@ -60,7 +60,7 @@ def test_argument_rejection_needs_no_gpu():
     assert need >= rows * 128 * 2 + 4 * rows * 4
     bargs = [p] * 5 + [p, p, p, p, p, p, p] + [p] * 6 + [p, need - 1, 2, 3, 256, 64, 0.125, 0.8, 1, None]
     assert lib.diffattn_backward(*bargs) == -4
-    bargs[19], bargs[-2] = need, 8
+    bargs[19], bargs[-2] = need, 16
     assert lib.diffattn_backward(*bargs) == -6
     for code in (0, -1, -2, -3, -4, -5, -6):
         assert len(lib.diffattn_strerror(code)) > 0
@@ -75,6 +75,8 @@ def test_host_validation_errors():
     t = lambda *s, dt=torch.float16: torch.zeros(*s, dtype=dt)
     with pytest.raises(TypeError):
         _check_inputs(t(1, 1, 128, 64, dt=torch.float32), *[t(1, 1, 128, 64)] * 3, t(1, 1, 128, 128))
+    with pytest.raises(TypeError):   # fp16 and bf16 inputs cannot be mixed
+        _check_inputs(t(1, 1, 128, 64, dt=torch.bfloat16), *[t(1, 1, 128, 64)] * 3, t(1, 1, 128, 128))
     with pytest.raises(ValueError):
         _check_inputs(t(1, 128, 64), *[t(1, 1, 128, 64)] * 3, t(1, 1, 128, 128))
     with pytest.raises(ValueError):  # CPU tensors are rejected: there is no CPU path

@@ -29,16 +29,17 @@ def test_scanner_flags_a_write_right_before_an_asm_mfma():
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
-def test_backward_kernels_have_no_unprotected_asm_mfma(tmp_path):
+@pytest.mark.parametrize("variant", [[], ["-DDA_BF16"]], ids=["fp16", "bf16"])
+def test_backward_kernels_have_no_unprotected_asm_mfma(tmp_path, variant):
     import importlib.util
     spec = importlib.util.spec_from_file_location("da_build", os.path.join(ROOT, "triton-diff-attn_amd", "build.py"))
     build = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(build)
     out = tmp_path / "bwd.s"
-    cmd = [build.HIPCC] + [f for f in build.FLAGS if f != "-fPIC"] + ["--cuda-device-only", "-S", "-o", str(out),
+    cmd = [build.HIPCC] + [f for f in build.FLAGS if f != "-fPIC"] + variant + ["--cuda-device-only", "-S", "-o", str(out),
                                                                           os.path.join(CSRC, "bwd.hip")]
     subprocess.run(cmd, check=True, capture_output=True)
     text = out.read_text()
-    assert "v_mfma_f32_32x32x16_f16" in text and ";;#ASMSTART" in text
+    assert ("v_mfma_f32_32x32x16_bf16" if variant else "v_mfma_f32_32x32x16_f16") in text and ";;#ASMSTART" in text
     hazards = isa_scan.asm_mfma_hazards(text)
     assert hazards == [], "VALU write right before an inline-asm MFMA: %s" % hazards[:5]

@@ -10,6 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdiffattn.so")
 SOURCES = ["fwd.hip", "bwd.hip", "api.hip"]
+KERNEL_SOURCES = ["fwd.hip", "bwd.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -23,9 +24,12 @@ FLAGS = [
 def build(verbose=True):
     objs = []
     procs = []
-    for src in SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-        cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    # the kernel sources are compiled twice: for fp16 tensors and, with -DDA_BF16, for bf16 tensors
+    units = [(src, [], src.replace(".hip", ".o")) for src in SOURCES]
+    units += [(src, ["-DDA_BF16"], src.replace(".hip", "_bf16.o")) for src in KERNEL_SOURCES]
+    for src, extra, obj_name in units:
+        obj = os.path.join(CSRC, obj_name)
+        cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

@@ -5,6 +5,15 @@
 
 using namespace da;
 
+// The bf16 build of the kernels (the same sources compiled with -DDA_BF16) lives in namespace da_bf16.
+// Its parameter blocks have the layout of the fp16 ones: pointers to 16-bit elements, ints, floats.
+namespace da_bf16 {
+struct FwdParams;
+struct BwdParams;
+hipError_t launch_fwd(const FwdParams& p, int D, hipStream_t stream);
+hipError_t launch_bwd(const BwdParams& p, int D, hipStream_t stream);
+}  // namespace da_bf16
+
 namespace {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -51,7 +60,7 @@ const char* diffattn_strerror(int code) {
     case DIFFATTN_EINVAL_SEQ: return "N must be a multiple of 128 (and 1 <= n_valid <= N)";
     case DIFFATTN_EINVAL_WS: return "workspace too small or misaligned";
     case DIFFATTN_EINVAL_ALIGN: return "tensor pointers must be 16-byte aligned";
-    case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL)";
+    case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL, DIFFATTN_BF16)";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -71,7 +80,7 @@ int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, cons
                             int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
                             void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y) return DIFFATTN_EINVAL_NULL;
-  if (flags & ~(DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL)) return DIFFATTN_EINVAL_FLAGS;
+  if (flags & ~(DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL | DIFFATTN_BF16)) return DIFFATTN_EINVAL_FLAGS;
   if (int e = check_dims(B, H, N, D)) return e;
   if (n_valid < 1 || n_valid > N) return DIFFATTN_EINVAL_SEQ;
   if (!aligned16(q1) || !aligned16(q2) || !aligned16(k1) || !aligned16(k2) || !aligned16(v) ||
@@ -83,6 +92,8 @@ int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, cons
   p.y = (half_t*)y; p.u2 = (half_t*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
   p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0; p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
   p.n_keys = n_valid;
+  if (flags & DIFFATTN_BF16)
+    return (int)da_bf16::launch_fwd(reinterpret_cast<const da_bf16::FwdParams&>(p), D, (hipStream_t)stream);
   return (int)launch_fwd(p, D, (hipStream_t)stream);
 }
 
@@ -101,7 +112,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy ||
       !dq1 || !dq2 || !dk1 || !dk2 || !dv || !dlambda || !workspace)
     return DIFFATTN_EINVAL_NULL;
-  if (flags & ~(DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL)) return DIFFATTN_EINVAL_FLAGS;
+  if (flags & ~(DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL | DIFFATTN_BF16)) return DIFFATTN_EINVAL_FLAGS;
   if ((flags & DIFFATTN_RMS_NORM) && !rinv) return DIFFATTN_EINVAL_NULL;
   if (int e = check_dims(B, H, N, D)) return e;
   const void* ptrs[] = {q1, q2, k1, k2, v, y, u2, dy, dq1, dq2, dk1, dk2, dv};
@@ -121,6 +132,8 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   p.dlam_part = (float*)(ws + w.part); p.n_part = bwd_num_partials(B * H, N, D);
   p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0; p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
   p.stages = stage_mask & DIFFATTN_STAGE_ALL;
+  if (flags & DIFFATTN_BF16)
+    return (int)da_bf16::launch_bwd(reinterpret_cast<const da_bf16::BwdParams&>(p), D, (hipStream_t)stream);
   return (int)launch_bwd(p, D, (hipStream_t)stream);
 }
 

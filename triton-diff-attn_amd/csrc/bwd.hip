@@ -17,7 +17,7 @@
 
 #include "params.hpp"
 
-namespace da {
+namespace DA_NS {
 
 constexpr int kPrepRows = 64;   // rows per workgroup of the preprocess kernel = one d(lambda) partial
 
@@ -740,4 +740,4 @@ hipError_t launch_bwd(const BwdParams& p, int D, hipStream_t stream) {
   }
 }
 
-}  // namespace da
+}  // namespace DA_NS

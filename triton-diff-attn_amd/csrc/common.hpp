@@ -12,12 +12,30 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-namespace da {
+// The sources are compiled twice into one library: as they stand for fp16 tensors (namespace da),
+// and with -DDA_BF16 for bf16 tensors (namespace da_bf16).  "half" in comments means the 16-bit
+// element type of the build; everything that differs between the two is in this header.
+#ifdef DA_BF16
+#define DA_NS da_bf16
+#define DA_MFMA_32x32x16 "v_mfma_f32_32x32x16_bf16"
+#else
+#define DA_NS da
+#define DA_MFMA_32x32x16 "v_mfma_f32_32x32x16_f16"
+#endif
 
+namespace DA_NS {
+
+#ifdef DA_BF16
+typedef __bf16 half_t;
+typedef __bf16 h2 __attribute__((ext_vector_type(2)));
+typedef __bf16 h4 __attribute__((ext_vector_type(4)));
+typedef __bf16 h8 __attribute__((ext_vector_type(8)));
+#else
 typedef _Float16 half_t;
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+#endif
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef float f4v __attribute__((ext_vector_type(4)));
 typedef __fp16 tr4 __attribute__((vector_size(8)));
@@ -30,7 +48,21 @@ constexpr float kEps = 1e-5f;
 #define DA_LDS __attribute__((address_space(3)))
 
 __device__ __forceinline__ f16v mfma32(h8 a, h8 b, f16v c) {
+#ifdef DA_BF16
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#else
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#endif
+}
+
+// acc + x[0]*1 + x[1]*1 in one instruction: the sum of two rounded 16-bit values in fp32
+__device__ __forceinline__ float add_pair(h2 x, float acc) {
+  const h2 ones = {(half_t)1.0f, (half_t)1.0f};
+#ifdef DA_BF16
+  return __builtin_amdgcn_fdot2_f32_bf16(x, ones, acc, false);
+#else
+  return __builtin_amdgcn_fdot2(x, ones, acc, false);
+#endif
 }
 
 // MFMA with the B operand held in an accumulation register (AGPR) and the result in ordinary
@@ -39,7 +71,7 @@ __device__ __forceinline__ f16v mfma32(h8 a, h8 b, f16v c) {
 // compiler does not know these are matrix instructions: the caller must put mfma_results_ready()
 // between the last of them and the first VALU read of the result.
 __device__ __forceinline__ f16v mfma32_bagpr(h8 a, h8 b, f16v c) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  asm volatile(DA_MFMA_32x32x16 " %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
   return c;
 }
 // Moves a fragment into AGPRs for good: after this the value is defined by an (empty) asm statement
@@ -77,7 +109,12 @@ __device__ __forceinline__ float pair_sum(float x) { LanePair p = lane_pair(x); 
 
 // 4x16 transposing LDS read (see header comment); p must be 8-byte aligned.
 __device__ __forceinline__ h4 lds_read_tr(const half_t* p) {
+#ifdef DA_BF16
+  typedef short tr4i __attribute__((ext_vector_type(4)));
+  tr4i v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DA_LDS tr4i*)(p));
+#else
   tr4 v = __builtin_amdgcn_ds_read_tr16_b64_v4f16((DA_LDS tr4*)(p));
+#endif
   return __builtin_bit_cast(h4, v);
 }
 
@@ -193,4 +230,4 @@ __device__ __forceinline__ int xcd_remap(int wg, int total) {
   return (wg % kXcd) * (total / kXcd) + wg / kXcd;
 }
 
-}  // namespace da
+}  // namespace DA_NS

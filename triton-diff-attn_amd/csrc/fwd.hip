@@ -14,7 +14,7 @@
 //     transposing LDS read, using the same key permutation as the accumulator layout.
 #include "params.hpp"
 
-namespace da {
+namespace DA_NS {
 
 template <int D>
 struct FwdCfg {
@@ -253,7 +253,6 @@ void fwd_kernel(FwdParams p) {
     scores(ka, s_nxt);
 
     h8 pb[QS][NKK];      // P^T as B operands: pb[kk] covers keys 16kk..16kk+15 (accumulator order)
-    const h2 ones = {(half_t)1.0f, (half_t)1.0f};
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
       float rs = 0.f;
@@ -264,7 +263,7 @@ void fwd_kernel(FwdParams p) {
           h2 e2;
           e2[0] = (half_t)fast_exp2(s_cur[qs][kt][r]);
           e2[1] = (half_t)fast_exp2(s_cur[qs][kt][r + 1]);
-          rs = __builtin_amdgcn_fdot2(e2, ones, rs, false);   // row sum of the rounded probabilities
+          rs = add_pair(e2, rs);   // row sum of the rounded probabilities
           pb[qs][kt * 2 + r / 8][r % 8] = e2[0];
           pb[qs][kt * 2 + r / 8][r % 8 + 1] = e2[1];
         }
@@ -404,4 +403,4 @@ hipError_t launch_fwd(const FwdParams& p, int D, hipStream_t stream) {
   }
 }
 
-}  // namespace da
+}  // namespace DA_NS

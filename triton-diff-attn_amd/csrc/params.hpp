@@ -3,7 +3,7 @@
 #include <hip/hip_runtime.h>
 #include "common.hpp"
 
-namespace da {
+namespace DA_NS {
 
 struct FwdParams {
   const half_t* q1; const half_t* q2; const half_t* k1; const half_t* k2; const half_t* v;
@@ -43,4 +43,4 @@ hipError_t launch_fwd(const FwdParams& p, int D, hipStream_t stream);
 hipError_t launch_bwd(const BwdParams& p, int D, hipStream_t stream);
 int bwd_num_partials(int BH, int N, int D);
 
-}  // namespace da
+}  // namespace DA_NS

@@ -14,6 +14,8 @@ _SUPPORTED_D = (32, 64, 128)
 _SEQ_MULTIPLE = 128
 _FLAG_RMS_NORM = 1      # DIFFATTN_RMS_NORM
 _FLAG_CAUSAL = 2        # DIFFATTN_CAUSAL
+_FLAG_BF16 = 4          # DIFFATTN_BF16
+_DTYPES = (torch.float16, torch.bfloat16)
 
 
 def _check_inputs(Q1, Q2, K1, K2, V):
@@ -21,11 +23,14 @@ def _check_inputs(Q1, Q2, K1, K2, V):
     for n, t in zip(names, (Q1, Q2, K1, K2, V)):
         if not torch.is_tensor(t):
             raise TypeError("%s must be a tensor" % n)
-        if t.dtype != torch.float16:
-            raise TypeError("%s must be float16 (got %s); the kernels are fp16-only like the reference "
-                            "(src/kernel.py:3-4)" % (n, t.dtype))
+        if t.dtype not in _DTYPES:
+            raise TypeError("%s must be float16 (like the reference, src/kernel.py:3-4) or bfloat16 (got %s)"
+                            % (n, t.dtype))
+        if t.dtype != Q1.dtype:
+            raise TypeError("all inputs must have the same dtype (%s has %s, q1 has %s)" % (n, t.dtype, Q1.dtype))
         if t.dim() != 4:
             raise ValueError("%s must be [B,H,N,D] (got %d dims)" % (n, t.dim()))
+    for n, t in zip(names, (Q1, Q2, K1, K2, V)):
         if not t.is_cuda:
             raise ValueError("%s must live on the GPU" % n)
         if t.device != Q1.device:
@@ -50,14 +55,14 @@ def _pad_rows(t, n_pad):
     return torch.nn.functional.pad(t, (0, 0, 0, n_pad - t.size(2)))
 
 
-def _lambda_tensor(lambda_scale, device):
-    """The kernels read lambda from device memory (src/kernel.py:138).  A python number is wrapped
-    (a superset of the reference, whose float default cannot reach its kernel)."""
+def _lambda_tensor(lambda_scale, device, dtype=torch.float16):
+    """The kernels read lambda from device memory (src/kernel.py:138), in the dtype of the tensors.  A
+    python number is wrapped (a superset of the reference, whose float default cannot reach its kernel)."""
     if torch.is_tensor(lambda_scale):
         if lambda_scale.numel() != 1:
             raise ValueError("lambda_scale must have exactly one element")
-        return lambda_scale.detach().to(device=device, dtype=torch.float16).reshape(1).contiguous()
-    return torch.tensor([float(lambda_scale)], dtype=torch.float16, device=device)
+        return lambda_scale.detach().to(device=device, dtype=dtype).reshape(1).contiguous()
+    return torch.tensor([float(lambda_scale)], dtype=dtype, device=device)
 
 
 def _ptr(t):
@@ -76,9 +81,10 @@ class _diff_attention(torch.autograd.Function):
         # k, v and upstream-gradient rows there the backward is exact on the real rows.
         n_pad = -(-N // _SEQ_MULTIPLE) * _SEQ_MULTIPLE
         q1, q2, k1, k2, v = (_pad_rows(t, n_pad) for t in (Q1, Q2, K1, K2, V))
-        lam = _lambda_tensor(LAMBDA_SCALE, dev)
+        lam = _lambda_tensor(LAMBDA_SCALE, dev, Q1.dtype)
         rms_norm = bool(rms_norm)
-        flags = (_FLAG_RMS_NORM if rms_norm else 0) | (_FLAG_CAUSAL if causal else 0)
+        flags = ((_FLAG_RMS_NORM if rms_norm else 0) | (_FLAG_CAUSAL if causal else 0)
+                 | (_FLAG_BF16 if Q1.dtype == torch.bfloat16 else 0))
 
         y = torch.empty_like(v)
         u2 = torch.empty_like(v)
@@ -107,15 +113,15 @@ class _diff_attention(torch.autograd.Function):
         B, H, N, D = q1.shape
         lib = _native.lib()
         dev = q1.device
-        if dO.dtype != torch.float16:
-            dO = dO.to(torch.float16)
+        if dO.dtype != q1.dtype:
+            dO = dO.to(q1.dtype)
         dO = _pad_rows(dO, N)           # N is the padded length here
         n_valid = ctx.N_VALID
 
         dq1, dq2 = torch.empty_like(q1), torch.empty_like(q2)
         dk1, dk2 = torch.empty_like(k1), torch.empty_like(k2)
         dv = torch.empty_like(v)
-        dlam = torch.empty(1, device=dev, dtype=torch.float16)
+        dlam = torch.empty(1, device=dev, dtype=q1.dtype)
         ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D)
         ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
 
