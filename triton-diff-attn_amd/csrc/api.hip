@@ -6,10 +6,9 @@
 using namespace da;
 
 // The bf16 build of the kernels (the same sources compiled with -DDA_BF16) lives in namespace da_bf16.
-// Its parameter blocks have the layout of the fp16 ones: pointers to 16-bit elements, ints, floats.
 namespace da_bf16 {
-struct FwdParams;
-struct BwdParams;
+using FwdParams = da_abi::FwdParamsT<__bf16>;
+using BwdParams = da_abi::BwdParamsT<__bf16>;
 hipError_t launch_fwd(const FwdParams& p, int D, hipStream_t stream);
 hipError_t launch_bwd(const BwdParams& p, int D, hipStream_t stream);
 }  // namespace da_bf16
@@ -44,6 +43,39 @@ WsLayout ws_layout(int BH, int N, int D) {
   w.part = off;    off = round_up(off + (size_t)bwd_num_partials(BH, N, D) * sizeof(float), 256);
   w.total = off;
   return w;
+}
+
+template <class T>
+void fill_fwd(da_abi::FwdParamsT<T>& p, const void* q1, const void* q2, const void* k1, const void* k2,
+              const void* v, const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
+              int BH, int N, int n_valid, float sm_scale, float lambda_init, int flags) {
+  p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
+  p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
+  p.y = (T*)y; p.u2 = (T*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
+  p.BH = BH; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init;
+  p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0;
+  p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
+  p.n_keys = n_valid;
+}
+
+template <class T>
+void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const void* k1, const void* k2,
+              const void* v, const void* lambda_scale, const void* y, const void* u2,
+              const float* lse1, const float* lse2, const float* rinv, const void* dy,
+              void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
+              void* ws_dx, void* ws_stat, void* ws_part, int n_part,
+              int BH, int N, float sm_scale, float lambda_init, int flags, unsigned stage_mask) {
+  p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
+  p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
+  p.y = (const T*)y; p.u2 = (const T*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
+  p.dy = (const T*)dy;
+  p.dq1 = (T*)dq1; p.dq2 = (T*)dq2; p.dk1 = (T*)dk1; p.dk2 = (T*)dk2; p.dv = (T*)dv;
+  p.dlambda = (T*)dlambda;
+  p.dx = (T*)ws_dx; p.stat = (float*)ws_stat; p.dlam_part = (float*)ws_part; p.n_part = n_part;
+  p.BH = BH; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init;
+  p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0;
+  p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
+  p.stages = stage_mask & DIFFATTN_STAGE_ALL;
 }
 
 }  // namespace
@@ -86,14 +118,13 @@ int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, cons
   if (!aligned16(q1) || !aligned16(q2) || !aligned16(k1) || !aligned16(k2) || !aligned16(v) ||
       !aligned16(y) || !aligned16(u2))
     return DIFFATTN_EINVAL_ALIGN;
+  if (flags & DIFFATTN_BF16) {
+    da_bf16::FwdParams p;
+    fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, N, n_valid, sm_scale, lambda_init, flags);
+    return (int)da_bf16::launch_fwd(p, D, (hipStream_t)stream);
+  }
   FwdParams p;
-  p.q1 = (const half_t*)q1; p.q2 = (const half_t*)q2; p.k1 = (const half_t*)k1; p.k2 = (const half_t*)k2;
-  p.v = (const half_t*)v; p.lambda_scale = (const half_t*)lambda_scale;
-  p.y = (half_t*)y; p.u2 = (half_t*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
-  p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0; p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
-  p.n_keys = n_valid;
-  if (flags & DIFFATTN_BF16)
-    return (int)da_bf16::launch_fwd(reinterpret_cast<const da_bf16::FwdParams&>(p), D, (hipStream_t)stream);
+  fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, N, n_valid, sm_scale, lambda_init, flags);
   return (int)launch_fwd(p, D, (hipStream_t)stream);
 }
 
@@ -121,19 +152,16 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   const WsLayout w = ws_layout(B * H, N, D);
   if (workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return DIFFATTN_EINVAL_WS;
   char* ws = (char*)workspace;
+  const int n_part = bwd_num_partials(B * H, N, D);
+  if (flags & DIFFATTN_BF16) {
+    da_bf16::BwdParams p;
+    fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
+             ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, N, sm_scale, lambda_init, flags, stage_mask);
+    return (int)da_bf16::launch_bwd(p, D, (hipStream_t)stream);
+  }
   BwdParams p;
-  p.q1 = (const half_t*)q1; p.q2 = (const half_t*)q2; p.k1 = (const half_t*)k1; p.k2 = (const half_t*)k2;
-  p.v = (const half_t*)v; p.lambda_scale = (const half_t*)lambda_scale;
-  p.y = (const half_t*)y; p.u2 = (const half_t*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
-  p.dy = (const half_t*)dy;
-  p.dq1 = (half_t*)dq1; p.dq2 = (half_t*)dq2; p.dk1 = (half_t*)dk1; p.dk2 = (half_t*)dk2; p.dv = (half_t*)dv;
-  p.dlambda = (half_t*)dlambda;
-  p.dx = (half_t*)(ws + w.dx); p.stat = (float*)(ws + w.stat);
-  p.dlam_part = (float*)(ws + w.part); p.n_part = bwd_num_partials(B * H, N, D);
-  p.BH = B * H; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init; p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0; p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
-  p.stages = stage_mask & DIFFATTN_STAGE_ALL;
-  if (flags & DIFFATTN_BF16)
-    return (int)da_bf16::launch_bwd(reinterpret_cast<const da_bf16::BwdParams&>(p), D, (hipStream_t)stream);
+  fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
+           ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, N, sm_scale, lambda_init, flags, stage_mask);
   return (int)launch_bwd(p, D, (hipStream_t)stream);
 }
 

@@ -507,6 +507,9 @@ struct DqCfg {
   // accumulators of a D = 128 wave do not fit 256 registers
   static constexpr int OCC = (D == 128) ? 1 : 2;
   static constexpr int NT = NW * 64;
+  // thread count the register budget is derived from: with fewer than 4 * OCC waves in a workgroup
+  // the occupancy attribute alone does not hold the allocator to 512 / OCC registers
+  static constexpr int REG_NT = (OCC * 256 > NT) ? OCC * 256 : NT;
   static constexpr int BM = NW * 32;           // query rows per workgroup
   static constexpr int BN = (D <= 64) ? 64 : 32;  // keys per staged tile
   static constexpr int K_TILE = BN * D;        // halfs (swizzled, unpadded)
@@ -519,7 +522,7 @@ struct DqCfg {
 // [keys x queries], so that a lane owns one query column: the row statistics are per-lane
 // scalars and dS^T in accumulator layout is directly the B operand of dQ^T = K^T dS^T.
 template <int D, int NWAVES, bool CAUSAL>
-__global__ __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(DqCfg<D, NWAVES>::OCC, DqCfg<D, NWAVES>::OCC))) void bwd_dq_kernel(BwdParams p) {
+__global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_waves_per_eu(DqCfg<D, NWAVES>::OCC, DqCfg<D, NWAVES>::OCC))) void bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<D, NWAVES>;
   constexpr int DV = C::DV, NW = C::NW, BM = C::BM, BN = C::BN;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
