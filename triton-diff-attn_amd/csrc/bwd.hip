@@ -150,8 +150,14 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   const int j = lane & 31, g = lane >> 5;
 
   const int n_kt = p.N / BK;
-  const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = tile / n_kt, kt = tile % n_kt;
+  int bh, kt;
+  if constexpr (CAUSAL) {   // the first key block of a unit is seen by the most queries
+    const UnitBlock ub = longest_first(blockIdx.x, p.BH);
+    bh = ub.unit; kt = ub.rank;
+  } else {
+    const int tile = xcd_remap(blockIdx.x, gridDim.x);
+    bh = tile / n_kt; kt = tile % n_kt;
+  }
   const size_t rows = (size_t)p.BH * p.N;
   const size_t row0 = (size_t)bh * p.N;
   const int key = kt * BK + wave * 32 + j;
@@ -534,9 +540,14 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   const int j = lane & 31, g = lane >> 5;
 
   const int n_qt = p.N / BM;
-  const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  // causal: the query blocks of a (batch, head) are visited last to first, longest loops first
-  const int bh = tile / n_qt, qt = CAUSAL ? (n_qt - 1 - tile % n_qt) : (tile % n_qt);
+  int bh, qt;
+  if constexpr (CAUSAL) {   // the last query block of a unit sees the most keys
+    const UnitBlock ub = longest_first(blockIdx.x, p.BH);
+    bh = ub.unit; qt = n_qt - 1 - ub.rank;
+  } else {
+    const int tile = xcd_remap(blockIdx.x, gridDim.x);
+    bh = tile / n_qt; qt = tile % n_qt;
+  }
   const size_t rows = (size_t)p.BH * p.N;
   const size_t row0 = (size_t)bh * p.N;
   const size_t qrow = row0 + qt * BM + wave * 32 + j;
@@ -722,10 +733,15 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
   if (p.stages & 8u) {
     // 256 query rows per workgroup when the sequence allows it, otherwise 128; a D = 128 workgroup
     // runs one wave per SIMD and therefore has four waves
-    if (p.N % 256 == 0 && D != 128) {
-      if (p.causal) hipLaunchKernelGGL((bwd_dq_kernel<D, 8, true>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
-      else          hipLaunchKernelGGL((bwd_dq_kernel<D, 8, false>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
-    } else {
+    bool wide = false;
+    if constexpr (D != 128) {
+      if (p.N % 256 == 0) {
+        wide = true;
+        if (p.causal) hipLaunchKernelGGL((bwd_dq_kernel<D, 8, true>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
+        else          hipLaunchKernelGGL((bwd_dq_kernel<D, 8, false>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
+      }
+    }
+    if (!wide) {
       if (p.causal) hipLaunchKernelGGL((bwd_dq_kernel<D, 4, true>), dim3(p.BH * (p.N / 128)), dim3(256), 0, stream, p);
       else          hipLaunchKernelGGL((bwd_dq_kernel<D, 4, false>), dim3(p.BH * (p.N / 128)), dim3(256), 0, stream, p);
     }

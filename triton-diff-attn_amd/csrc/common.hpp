@@ -232,4 +232,14 @@ __device__ __forceinline__ int xcd_remap(int wg, int total) {
   return (wg % kXcd) * (total / kXcd) + wg / kXcd;
 }
 
+// Workgroup id -> (batch*head unit, rank of the block inside the unit) for kernels whose blocks
+// differ in length (causal mask).  Workgroups are dispatched in id order, so all units' blocks of
+// rank 0 come first, then rank 1, ...: with rank 0 the longest loop this is longest-first list
+// scheduling over the whole grid, which keeps the CUs evenly loaded to the end.  Unit = id % BH
+// also keeps a unit on one XCD whenever BH is a multiple of 8.
+struct UnitBlock { int unit, rank; };
+__device__ __forceinline__ UnitBlock longest_first(int wg, int n_units) {
+  return {wg % n_units, wg / n_units};
+}
+
 }  // namespace DA_NS

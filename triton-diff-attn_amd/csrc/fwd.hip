@@ -60,10 +60,15 @@ void fwd_kernel(FwdParams p) {
   const int j = lane & 31, g = lane >> 5;
 
   const int n_qt = p.N / BM;
-  const int tile = xcd_remap(blockIdx.x, gridDim.x);
-  // causal: the query blocks of a (batch, head) are visited last to first, longest loops first
   constexpr bool CAUSAL = (MASK == 1), PADDED = (MASK == 2);
-  const int bh = tile / n_qt, qt = CAUSAL ? (n_qt - 1 - tile % n_qt) : (tile % n_qt);
+  int bh, qt;
+  if constexpr (CAUSAL) {   // the last query block of a unit sees the most keys
+    const UnitBlock ub = longest_first(blockIdx.x, p.BH);
+    bh = ub.unit; qt = n_qt - 1 - ub.rank;
+  } else {
+    const int tile = xcd_remap(blockIdx.x, gridDim.x);
+    bh = tile / n_qt; qt = tile % n_qt;
+  }
   const size_t qk_base = (size_t)bh * p.N * D;
   const size_t v_base = (size_t)bh * p.N * DV;
   const int qrow0 = qt * BM + qw * 32 * QS + j;   // this lane's query row of block qs is qrow0 + 32*qs
