@@ -12,7 +12,7 @@
  *     gradients, [B,H,N,2D] for v, y, u2, dy, dv; row statistics are fp32 [B,H,N];
  *   - D is 32, 64 or 128; N is a multiple of 128;
  *   - lambda_scale is a DEVICE pointer to one fp16 value (the reference loads it in-kernel,
- *     src/kernel.py:138);
+ *     src/kernel.py:138), or to H values with DIFFATTN_LAMBDA_PER_HEAD;
  *   - `stream` is a hipStream_t passed as void*; work is only enqueued on it.  No entry point
  *     allocates, frees, synchronises or keeps global state; all are re-entrant;
  *   - return value: 0 on success, a negative DIFFATTN_E* code for rejected arguments, or a
@@ -45,6 +45,10 @@ extern "C" {
 /* Every 16-bit tensor (q1..v, y, u2, dy, the gradients, *lambda_scale, *dlambda) is bfloat16 instead of
  * fp16.  No counterpart in the reference, whose kernel hard-codes fp16 (src/kernel.py:175-176). */
 #define DIFFATTN_BF16 4
+/* lambda_scale points to H values, one per head (head h of every batch entry uses lambda_scale[h]), and
+ * the backward writes H values to dlambda, each summed over the batch.  No counterpart in the
+ * reference, which has one lambda per call (src/kernel.py:138). */
+#define DIFFATTN_LAMBDA_PER_HEAD 8
 
 /* ABI version of this header; bumped when a signature changes. */
 int diffattn_abi_version(void);
@@ -89,8 +93,9 @@ size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D);
  * reduction of the lambda gradient (src/kernel.py:573).
  *   inputs : q1,q2,k1,k2,v,lambda_scale as in forward; y,u2,lse1,lse2,rinv as written by forward
  *            (rinv is ignored without DIFFATTN_RMS_NORM); dy [B,H,N,2D] upstream gradient, dense.
- *   outputs: dq1,dq2,dk1,dk2 [B,H,N,D], dv [B,H,N,2D] fp16; dlambda: one fp16 value, DEVICE
- *            memory, written (not accumulated), reduced in a fixed order: bit-reproducible.
+ *   outputs: dq1,dq2,dk1,dk2 [B,H,N,D], dv [B,H,N,2D] fp16; dlambda: one fp16 value (H values
+ *            with DIFFATTN_LAMBDA_PER_HEAD), DEVICE memory, written (not accumulated), reduced in
+ *            a fixed order: bit-reproducible.
  *   workspace: device memory of at least diffattn_backward_workspace_bytes(B,H,N,D) bytes,
  *            256-byte aligned, contents undefined before and after.
  */

@@ -33,6 +33,23 @@ def _as_scalar(lambda_scale, dtype):
     return torch.tensor(float(lambda_scale), dtype=dtype)
 
 
+def _lambda_values(lambda_scale, H, dtype):
+    """lambda as a vector: one value (the reference's case, src/layers.py:70) or one per head (not in
+    the reference: each head then has its own lambda, shared over the batch)."""
+    if torch.is_tensor(lambda_scale) and lambda_scale.numel() > 1:
+        if lambda_scale.numel() != H:
+            raise ValueError("lambda_scale must have 1 or H elements")
+        return lambda_scale.reshape(H).to(dtype)
+    return _as_scalar(lambda_scale, dtype).reshape(1)
+
+
+def _lambda_of_units(lam_values, units, H):
+    """[len(units), 1, 1] lambda of the (batch, head) units `units` (unit = b * H + h)."""
+    if lam_values.numel() == 1:
+        return lam_values.reshape(1, 1, 1)
+    return lam_values[units % H].reshape(-1, 1, 1)
+
+
 def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False, causal=False):
     """One or more (b, h) units: tensors [..., N, D] / [..., N, 2D], already in the work dtype.
 
@@ -83,10 +100,11 @@ def forward(q1, q2, k1, k2, v, lambda_scale, lambda_init=0.8, rms_norm=False,
     Dv = v.shape[-1]
     f = lambda t: t.reshape(B * H, N, t.shape[-1]).to(dtype)
     q1f, q2f, k1f, k2f, vf = f(q1), f(q2), f(k1), f(k2), f(v)
-    lam = _as_scalar(lambda_scale, dtype)
+    lam_values = _lambda_values(lambda_scale, H, dtype)
     ys, auxs = [], []
     for s in range(0, B * H, chunk):
         sl = slice(s, s + chunk)
+        lam = _lambda_of_units(lam_values, torch.arange(s, min(s + chunk, B * H)), H)
         r = forward_unit(q1f[sl], q2f[sl], k1f[sl], k2f[sl], vf[sl], lam, lambda_init, rms_norm, want_aux, causal)
         if want_aux:
             ys.append(r[0]); auxs.append(r[1])
@@ -111,30 +129,31 @@ def forward_backward(q1, q2, k1, k2, v, lambda_scale, dy, lambda_init=0.8, rms_n
 
     Returns (y, dq1, dq2, dk1, dk2, dv, dlambda) in `dtype`; dlambda has shape [1] and is the sum
     over all (b,h) units (the reference sums its per-program partials the same way,
-    src/kernel.py:573).
+    src/kernel.py:573).  With one lambda per head, dlambda has shape [H]: the sum over the batch.
     """
     B, H, N, D = q1.shape
     Dv = v.shape[-1]
     f = lambda t: t.reshape(B * H, N, t.shape[-1]).to(dtype)
     ins = [f(q1), f(q2), f(k1), f(k2), f(v)]
     dyf = f(dy)
-    lam0 = _as_scalar(lambda_scale, dtype)
+    lam0 = _lambda_values(lambda_scale, H, dtype)
     grads = [torch.empty_like(t) for t in ins]
-    dlam = torch.zeros((), dtype=dtype)
+    dlam = torch.zeros_like(lam0)
     ys = []
     for s in range(0, B * H, chunk):
         sl = slice(s, s + chunk)
         leaves = [t[sl].detach().clone().requires_grad_(True) for t in ins]
-        lam = lam0.detach().clone().requires_grad_(True)
+        lam_leaf = lam0.detach().clone().requires_grad_(True)
+        lam = _lambda_of_units(lam_leaf, torch.arange(s, min(s + chunk, B * H)), H)
         y = forward_unit(*leaves, lam, lambda_init, rms_norm, causal=causal)
-        g = torch.autograd.grad(y, leaves + [lam], dyf[sl])
+        g = torch.autograd.grad(y, leaves + [lam_leaf], dyf[sl])
         for dst, src in zip(grads, g[:5]):
             dst[sl] = src
         dlam = dlam + g[5]
         ys.append(y.detach())
     y = torch.cat(ys).reshape(B, H, N, Dv)
     shp = lambda t: t.reshape(B, H, N, t.shape[-1])
-    return (y, shp(grads[0]), shp(grads[1]), shp(grads[2]), shp(grads[3]), shp(grads[4]), dlam.reshape(1))
+    return (y, shp(grads[0]), shp(grads[1]), shp(grads[2]), shp(grads[3]), shp(grads[4]), dlam)
 
 
 def backward_explicit(q1, q2, k1, k2, v, lambda_scale, dy, lambda_init=0.8, rms_norm=False,

@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_symbols():
         assert hasattr(lib, name), name
         assert name in _native.SYMBOLS, "binding table misses %s" % name
-    assert lib.diffattn_abi_version() == 2
+    assert lib.diffattn_abi_version() == 3
 
 
 def test_argument_rejection_needs_no_gpu():
@@ -48,7 +48,7 @@ def test_argument_rejection_needs_no_gpu():
     bad[0] = p + 2
     assert lib.diffattn_forward(*bad) == -5
     bad = args(1, 1, 128, 64)
-    bad[-2] = 8                                   # unknown flag bit
+    bad[-2] = 16                                  # unknown flag bit
     assert lib.diffattn_forward(*bad) == -6
     padded = lambda n_valid: [p] * 11 + [1, 1, 128, n_valid, 64, 0.125, 0.8, 1, None]
     assert lib.diffattn_forward_padded(*padded(0)) == -3
@@ -60,7 +60,7 @@ def test_argument_rejection_needs_no_gpu():
     assert need >= rows * 128 * 2 + 4 * rows * 4
     bargs = [p] * 5 + [p, p, p, p, p, p, p] + [p] * 6 + [p, need - 1, 2, 3, 256, 64, 0.125, 0.8, 1, None]
     assert lib.diffattn_backward(*bargs) == -4
-    bargs[19], bargs[-2] = need, 16
+    bargs[19], bargs[-2] = need, 32
     assert lib.diffattn_backward(*bargs) == -6
     for code in (0, -1, -2, -3, -4, -5, -6):
         assert len(lib.diffattn_strerror(code)) > 0
@@ -83,6 +83,10 @@ def test_host_validation_errors():
         _check_inputs(*[t(1, 1, 128, 64)] * 4, t(1, 1, 128, 128))
     with pytest.raises(ValueError):
         _lambda_tensor(torch.zeros(2), torch.device("cpu"))
+    with pytest.raises(ValueError):   # neither one value nor one per head
+        _lambda_tensor(torch.zeros(3), torch.device("cpu"), num_heads=4)
+    per_head = _lambda_tensor(torch.tensor([[0.1], [0.2], [0.3]]), torch.device("cpu"), num_heads=3)
+    assert per_head.shape == (3,) and per_head.dtype == torch.float16
     from kernel import _pad_rows
     x = torch.arange(2 * 3 * 5 * 4, dtype=torch.float16).reshape(2, 3, 5, 4)
     padded = _pad_rows(x, 8)

@@ -86,3 +86,46 @@ def test_causal_layer_with_the_kernel_matches_the_stock_operator():
     # a causal layer's output at position i does not change when later positions do
     x2 = x.clone(); x2[:, 200:] = 0
     assert (fused(x2)[:, :200].float() - y_f[:, :200].float()).abs().max().item() <= 2e-3
+
+
+def test_per_head_lambda_layer():
+    torch.manual_seed(4)
+    one = modules.DiffAttn(64, 4, depth=2, attention=baselines.MultiheadDiffAttn, dtype=torch.float32)
+    per = modules.DiffAttn(64, 4, depth=2, attention=baselines.MultiheadDiffAttn, per_head_lambda=True,
+                           dtype=torch.float32)
+    assert per.lambda_q1.shape == (4, 8) and per.lambda_scale().shape == (4,)
+    # with every head given the single-lambda layer's vectors, the two layers are the same function
+    state = one.state_dict()
+    for name in ("lambda_q1", "lambda_k1", "lambda_q2", "lambda_k2"):
+        state[name] = state[name].expand(4, -1).clone()
+    per.load_state_dict(state)
+    x = torch.randn(2, 12, 64)
+    assert torch.allclose(per(x), one(x), atol=1e-6)
+    # distinct per-head vectors give distinct lambdas, and each reaches the output
+    with torch.no_grad():
+        per.lambda_q1.copy_(torch.linspace(-0.5, 0.5, 32).reshape(4, 8))
+    lam = per.lambda_scale()
+    assert lam.unique().numel() == 4
+    per(x).square().mean().backward()
+    assert per.lambda_q1.grad.abs().sum(-1).min() > 0
+
+
+@pytest.mark.gpu
+def test_per_head_lambda_layer_with_the_kernel_matches_the_stock_operator():
+    torch.manual_seed(5)
+    dev = torch.device("cuda:0")
+    fused = modules.DiffAttn(512, 4, depth=3, per_head_lambda=True, device=dev)
+    with torch.no_grad():
+        fused.lambda_q1.copy_(torch.linspace(-0.3, 0.3, 4 * 64).reshape(4, 64))
+    stock = copy.deepcopy(fused)
+    stock.attention = baselines.MultiheadDiffAttn
+    x = (0.5 * torch.randn(2, 256, 512, device=dev)).half()
+    xs = [x.clone().requires_grad_(True) for _ in range(2)]
+    ys = [m(xi) for m, xi in zip((fused, stock), xs)]
+    assert (ys[0].float() - ys[1].float()).abs().max().item() <= 1e-2
+    g = torch.randn_like(ys[0])
+    for y in ys:
+        y.backward(g)
+    for (name, pf), (_, ps) in zip(fused.named_parameters(), stock.named_parameters()):
+        scale = ps.grad.float().abs().max().item()
+        assert (pf.grad.float() - ps.grad.float()).abs().max().item() <= 5e-2 * scale + 1e-3, name

@@ -182,3 +182,26 @@ def test_causal_gradients_do_not_flow_from_the_past_to_future_keys():
     for g in (out[3], out[4], out[5]):          # dk1, dk2, dv of keys 10.. are exactly zero
         assert g[:, :, 10:].abs().max().item() == 0.0
     assert out[3][:, :, :10].abs().max().item() > 0
+
+
+def test_per_head_lambda_is_the_scalar_oracle_head_by_head():
+    """One lambda per head (not in the reference): head h of the result, its gradients and d(lambda)[h]
+    must be what the single-lambda oracle gives on that head alone, for every batch entry together."""
+    B, H, N, D = 2, 3, 24, 8
+    g = torch.Generator().manual_seed(11)
+    mk = lambda d: torch.randn(B, H, N, d, generator=g, dtype=torch.float64)
+    q1, q2, k1, k2, v, dy = mk(D), mk(D), mk(D), mk(D), mk(2 * D), mk(2 * D)
+    lam = torch.tensor([0.3, -0.7, 1.2], dtype=torch.float64)
+    for rms in (False, True):
+        for causal in (False, True):
+            full = orc.forward_backward(q1, q2, k1, k2, v, lam, dy, 0.8, rms, dtype=torch.float64, chunk=4, causal=causal)
+            assert full[6].shape == (H,)
+            y_fwd = orc.forward(q1, q2, k1, k2, v, lam, 0.8, rms, dtype=torch.float64, chunk=5, causal=causal)
+            assert torch.allclose(y_fwd, full[0], rtol=0, atol=1e-12)
+            for h in range(H):
+                sl = (slice(None), slice(h, h + 1))
+                one = orc.forward_backward(q1[sl], q2[sl], k1[sl], k2[sl], v[sl], lam[h], dy[sl], 0.8, rms,
+                                           dtype=torch.float64, chunk=1, causal=causal)
+                for a, b in zip(full[:6], one[:6]):
+                    assert torch.allclose(a[sl], b, rtol=0, atol=1e-12)
+                assert torch.allclose(full[6][h], one[6][0], rtol=1e-12, atol=1e-12)

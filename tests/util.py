@@ -32,7 +32,9 @@ def run_kernel(q1, q2, k1, k2, v, lam_value, lambda_init, rms_norm, dy=None, dev
 
     need = dy is not None
     t = [x.to(device).requires_grad_(need) for x in (q1, q2, k1, k2, v)]
-    lam = torch.tensor([lam_value], dtype=q1.dtype, device=device, requires_grad=need)
+    # one lambda, or a list with one per head
+    lam = torch.tensor(list(lam_value) if isinstance(lam_value, (list, tuple)) else [lam_value],
+                       dtype=q1.dtype, device=device, requires_grad=need)
     extra = {"causal": True} if causal else {}
     y = MultiheadDiffAttnKernel(*t, lambda_scale=lam, lambda_init=lambda_init, rms_norm=rms_norm, **extra)
     grads = None

@@ -27,6 +27,13 @@ def _rms(x: torch.Tensor) -> torch.Tensor:
     return F.rms_norm(x, (x.size(-1),), eps=RMS_EPS)
 
 
+def _per_head(lambda_scale):
+    """A lambda tensor with one value per head broadcasts over [B, H, N, *]; one value or a number stays."""
+    if torch.is_tensor(lambda_scale) and lambda_scale.numel() > 1:
+        return lambda_scale.reshape(1, -1, 1, 1)
+    return lambda_scale
+
+
 def _probabilities(q: torch.Tensor, k: torch.Tensor, causal: bool = False) -> torch.Tensor:
     """softmax(q k^T / sqrt(d)) with the softmax in fp32 and the result back in the input dtype."""
     scores = (q @ k.transpose(-1, -2)) * (1.0 / math.sqrt(q.size(-1)))
@@ -43,7 +50,7 @@ def MultiheadAttn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, rms_norm: b
 
 def MultiheadDiffAttn(q1, q2, k1, k2, v, lambda_scale=-0.5, lambda_init: float = 0.8, rms_norm: bool = False,
                       causal: bool = False):
-    weights = _probabilities(q1, k1, causal) - lambda_scale * _probabilities(q2, k2, causal)
+    weights = _probabilities(q1, k1, causal) - _per_head(lambda_scale) * _probabilities(q2, k2, causal)
     out = weights @ v
     if rms_norm:
         out = (1 - lambda_init) * _rms(out)
@@ -61,7 +68,7 @@ def MultiheadFlashDiffAttn(q1, q2, k1, k2, v, lambda_scale=-0.5, lambda_init: fl
     halves = v.split(q1.size(-1), dim=-1)
     stream1 = torch.cat([F.scaled_dot_product_attention(q1, k1, h, is_causal=causal) for h in halves], dim=-1)
     stream2 = torch.cat([F.scaled_dot_product_attention(q2, k2, h, is_causal=causal) for h in halves], dim=-1)
-    out = stream1 - lambda_scale * stream2
+    out = stream1 - _per_head(lambda_scale) * stream2
     if rms_norm:
         out = (1 - lambda_init) * _rms(out)
     return out

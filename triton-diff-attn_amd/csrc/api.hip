@@ -15,6 +15,8 @@ hipError_t launch_bwd(const BwdParams& p, int D, hipStream_t stream);
 
 namespace {
 
+constexpr int kKnownFlags = DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL | DIFFATTN_BF16 | DIFFATTN_LAMBDA_PER_HEAD;
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 int check_dims(int B, int H, int N, int D) {
@@ -48,7 +50,7 @@ WsLayout ws_layout(int BH, int N, int D) {
 template <class T>
 void fill_fwd(da_abi::FwdParamsT<T>& p, const void* q1, const void* q2, const void* k1, const void* k2,
               const void* v, const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
-              int BH, int N, int n_valid, float sm_scale, float lambda_init, int flags) {
+              int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags) {
   p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
   p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
   p.y = (T*)y; p.u2 = (T*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
@@ -56,6 +58,7 @@ void fill_fwd(da_abi::FwdParamsT<T>& p, const void* q1, const void* q2, const vo
   p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0;
   p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
   p.n_keys = n_valid;
+  p.H = H; p.lambda_stride = (flags & DIFFATTN_LAMBDA_PER_HEAD) ? 1 : 0;
 }
 
 template <class T>
@@ -64,7 +67,7 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
               const float* lse1, const float* lse2, const float* rinv, const void* dy,
               void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
               void* ws_dx, void* ws_stat, void* ws_part, int n_part,
-              int BH, int N, float sm_scale, float lambda_init, int flags, unsigned stage_mask) {
+              int BH, int H, int N, float sm_scale, float lambda_init, int flags, unsigned stage_mask) {
   p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
   p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
   p.y = (const T*)y; p.u2 = (const T*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
@@ -76,13 +79,14 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
   p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0;
   p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
   p.stages = stage_mask & DIFFATTN_STAGE_ALL;
+  p.H = H; p.lambda_stride = (flags & DIFFATTN_LAMBDA_PER_HEAD) ? 1 : 0;
 }
 
 }  // namespace
 
 extern "C" {
 
-int diffattn_abi_version(void) { return 2; }
+int diffattn_abi_version(void) { return 3; }
 
 const char* diffattn_strerror(int code) {
   switch (code) {
@@ -92,7 +96,7 @@ const char* diffattn_strerror(int code) {
     case DIFFATTN_EINVAL_SEQ: return "N must be a multiple of 128 (and 1 <= n_valid <= N)";
     case DIFFATTN_EINVAL_WS: return "workspace too small or misaligned";
     case DIFFATTN_EINVAL_ALIGN: return "tensor pointers must be 16-byte aligned";
-    case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL, DIFFATTN_BF16)";
+    case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL, DIFFATTN_BF16, DIFFATTN_LAMBDA_PER_HEAD)";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -112,7 +116,7 @@ int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, cons
                             int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
                             void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y) return DIFFATTN_EINVAL_NULL;
-  if (flags & ~(DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL | DIFFATTN_BF16)) return DIFFATTN_EINVAL_FLAGS;
+  if (flags & ~kKnownFlags) return DIFFATTN_EINVAL_FLAGS;
   if (int e = check_dims(B, H, N, D)) return e;
   if (n_valid < 1 || n_valid > N) return DIFFATTN_EINVAL_SEQ;
   if (!aligned16(q1) || !aligned16(q2) || !aligned16(k1) || !aligned16(k2) || !aligned16(v) ||
@@ -120,11 +124,11 @@ int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, cons
     return DIFFATTN_EINVAL_ALIGN;
   if (flags & DIFFATTN_BF16) {
     da_bf16::FwdParams p;
-    fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, N, n_valid, sm_scale, lambda_init, flags);
+    fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags);
     return (int)da_bf16::launch_fwd(p, D, (hipStream_t)stream);
   }
   FwdParams p;
-  fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, N, n_valid, sm_scale, lambda_init, flags);
+  fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags);
   return (int)launch_fwd(p, D, (hipStream_t)stream);
 }
 
@@ -143,7 +147,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy ||
       !dq1 || !dq2 || !dk1 || !dk2 || !dv || !dlambda || !workspace)
     return DIFFATTN_EINVAL_NULL;
-  if (flags & ~(DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL | DIFFATTN_BF16)) return DIFFATTN_EINVAL_FLAGS;
+  if (flags & ~kKnownFlags) return DIFFATTN_EINVAL_FLAGS;
   if ((flags & DIFFATTN_RMS_NORM) && !rinv) return DIFFATTN_EINVAL_NULL;
   if (int e = check_dims(B, H, N, D)) return e;
   const void* ptrs[] = {q1, q2, k1, k2, v, y, u2, dy, dq1, dq2, dk1, dk2, dv};
@@ -156,12 +160,12 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   if (flags & DIFFATTN_BF16) {
     da_bf16::BwdParams p;
     fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
-             ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, N, sm_scale, lambda_init, flags, stage_mask);
+             ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, sm_scale, lambda_init, flags, stage_mask);
     return (int)da_bf16::launch_bwd(p, D, (hipStream_t)stream);
   }
   BwdParams p;
   fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
-           ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, N, sm_scale, lambda_init, flags, stage_mask);
+           ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, sm_scale, lambda_init, flags, stage_mask);
   return (int)launch_bwd(p, D, (hipStream_t)stream);
 }
 

@@ -9,7 +9,7 @@
 //                     dV += (P1 - lambda P2)^T dX, dK_t += s dS_t^T Q_t      (:410-424)
 //   bwd_dq_kernel     one workgroup per 128 queries, loops over all key tiles:
 //                     dQ_t += s dS_t K_t                                      (:426-436)
-//   bwd_dlambda_kernel  fixed-order sum of the partials into one fp16 value   (:573)
+//   bwd_dlambda_kernel  fixed-order sum of the partials into one fp16 value (one per head with per-head lambda)   (:573)
 //
 // The pre-norm row X is rebuilt as Y / ((1 - lambda_init) * rinv); only U2 = softmax(S2) V is
 // needed besides it, because U1 = X + lambda U2.
@@ -29,7 +29,8 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
   constexpr int DV = 2 * D, LPR = DV / 8, RPP = 256 / LPR;
   __shared__ float red[256];
   const int tid = threadIdx.x, sub = tid % LPR, rloc = tid / LPR;
-  const float lam = (float)p.lambda_scale[0];
+  // the 64 rows of a workgroup belong to one (batch, head) unit: N is a multiple of 128
+  const float lam = da_abi::lambda_of_unit(p, (int)(((size_t)blockIdx.x * kPrepRows) / p.N));
   const float c = 1.0f - p.lambda_init;
   const size_t rows = (size_t)p.BH * p.N;
   float part = 0.f;
@@ -97,11 +98,20 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
   if (tid == 0) p.dlam_part[blockIdx.x] = red[0];
 }
 
-__global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restrict__ part, int n, half_t* out) {
+// Workgroup o of n_out sums the partials of the units o, o + n_out, o + 2 n_out, ...: with n_out = 1
+// every unit (one lambda), with n_out = H the units of head o (one lambda per head).  `per_unit`
+// consecutive partials belong to a unit.
+__global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restrict__ part, int per_unit, int n_units,
+                                                          half_t* out) {
   __shared__ float red[256];
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, o = blockIdx.x, n_out = gridDim.x;
+  const int n = (n_units / n_out) * per_unit;        // partials this workgroup sums
   float acc = 0.f;
-  for (int i = tid; i < n; i += 256) acc += part[i];
+  if (n_out == 1) {
+    for (int i = tid; i < n; i += 256) acc += part[i];
+  } else {
+    for (int i = tid; i < n; i += 256) acc += part[(size_t)(o + (i / per_unit) * n_out) * per_unit + i % per_unit];
+  }
   red[tid] = acc;
   __syncthreads();
 #pragma unroll
@@ -109,7 +119,7 @@ __global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restric
     if (tid < s) red[tid] += red[tid + s];
     __syncthreads();
   }
-  if (tid == 0) out[0] = (half_t)red[0];
+  if (tid == 0) out[o] = (half_t)red[0];
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -163,7 +173,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   const int key = kt * BK + wave * 32 + j;
 
   const float c = p.sm_scale * kLog2e;
-  const float lam = (float)p.lambda_scale[0];
+  const float lam = da_abi::lambda_of_unit(p, bh);
 
   // persistent B operands: this lane's key row of K1, K2, V
   h8 kf1[NKS], kf2[NKS], vf[NKV];
@@ -552,7 +562,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   const size_t row0 = (size_t)bh * p.N;
   const size_t qrow = row0 + qt * BM + wave * 32 + j;
 
-  const float lam = (float)p.lambda_scale[0];
+  const float lam = da_abi::lambda_of_unit(p, bh);
 
   // persistent B operands: this lane's query row of Q1, Q2 (pre-multiplied by sm_scale*log2(e)
   // exactly as in the forward kernel, so the recomputed probabilities match it), dX, and its row
@@ -713,7 +723,8 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 2u) {
-    hipLaunchKernelGGL(bwd_dlambda_kernel, dim3(1), dim3(256), 0, stream, p.dlam_part, n_prep, p.dlambda);
+    hipLaunchKernelGGL(bwd_dlambda_kernel, dim3(p.lambda_stride ? p.H : 1), dim3(256), 0, stream,
+                       p.dlam_part, n_prep / p.BH, p.BH, p.dlambda);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 4u) {

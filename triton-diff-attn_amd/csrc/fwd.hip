@@ -349,7 +349,7 @@ void fwd_kernel(FwdParams p) {
   if (st == 1) {
     if (p.u2) store_rows(p.u2 + wave_row0 * DV);
   } else {
-    const float lam = (float)p.lambda_scale[0];
+    const float lam = da_abi::lambda_of_unit(p, bh);
     const half_t* stg_u2 = smem + (size_t)(wave + NW / 2) * 32 * SROW;
     float ss = 0.f;
 #pragma unroll

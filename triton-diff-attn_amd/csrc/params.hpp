@@ -9,7 +9,7 @@ namespace da_abi {
 template <class T>
 struct FwdParamsT {
   const T* q1; const T* q2; const T* k1; const T* k2; const T* v;
-  const T* lambda_scale;        // 1-element device tensor
+  const T* lambda_scale;        // device memory: one value, or one per head (lambda_stride = 1)
   T* y;                         // [B,H,N,2D]
   T* u2;                        // [B,H,N,2D]  softmax(S2) V, saved for backward (may be null)
   float* lse1; float* lse2;     // [B,H,N] natural-log row logsumexp of the scaled scores (may be null)
@@ -19,17 +19,19 @@ struct FwdParamsT {
   int rms_norm;
   int causal;                   // query i sees keys 0..i only
   int n_keys;                   // keys n_keys..N-1 are padding and are ignored (N when there is none)
+  int H;                        // heads per batch entry: unit bh belongs to head bh % H
+  int lambda_stride;            // 0: lambda_scale[0] for every head; 1: lambda_scale[head]
 };
 
 template <class T>
 struct BwdParamsT {
   const T* q1; const T* q2; const T* k1; const T* k2; const T* v;
-  const T* lambda_scale;
+  const T* lambda_scale;        // one value, or one per head (lambda_stride = 1)
   const T* y; const T* u2;
   const float* lse1; const float* lse2; const float* rinv;
   const T* dy;
   T* dq1; T* dq2; T* dk1; T* dk2; T* dv;
-  T* dlambda;                   // 1 element
+  T* dlambda;                   // 1 element, or H elements with lambda_stride = 1
   // workspace carve-up
   T* dx;                        // [BH,N,2D] gradient w.r.t. the pre-norm rows, 16-bit
   float* stat;                  // [4][BH*N]: -lse1*log2(e), -lse2*log2(e), -delta1, -(lambda*delta1 + delta2)
@@ -40,7 +42,15 @@ struct BwdParamsT {
   int rms_norm;
   int causal;
   unsigned stages;              // bit 0 row preprocess, 1 d(lambda) reduce, 2 dK/dV, 3 dQ
+  int H;                        // heads per batch entry: unit bh belongs to head bh % H
+  int lambda_stride;            // 0: one lambda; 1: one per head
 };
+
+// lambda of the (batch, head) unit bh
+template <class P>
+__device__ __forceinline__ float lambda_of_unit(const P& p, int bh) {
+  return (float)p.lambda_scale[(bh % p.H) * p.lambda_stride];
+}
 
 }  // namespace da_abi
 

@@ -15,6 +15,7 @@ _SEQ_MULTIPLE = 128
 _FLAG_RMS_NORM = 1      # DIFFATTN_RMS_NORM
 _FLAG_CAUSAL = 2        # DIFFATTN_CAUSAL
 _FLAG_BF16 = 4          # DIFFATTN_BF16
+_FLAG_LAMBDA_PER_HEAD = 8   # DIFFATTN_LAMBDA_PER_HEAD
 _DTYPES = (torch.float16, torch.bfloat16)
 
 
@@ -55,13 +56,14 @@ def _pad_rows(t, n_pad):
     return torch.nn.functional.pad(t, (0, 0, 0, n_pad - t.size(2)))
 
 
-def _lambda_tensor(lambda_scale, device, dtype=torch.float16):
+def _lambda_tensor(lambda_scale, device, dtype=torch.float16, num_heads=1):
     """The kernels read lambda from device memory (src/kernel.py:138), in the dtype of the tensors.  A
-    python number is wrapped (a superset of the reference, whose float default cannot reach its kernel)."""
+    python number is wrapped (a superset of the reference, whose float default cannot reach its kernel).
+    A tensor holds one value, like the reference's, or one per head (`num_heads` values, more than one)."""
     if torch.is_tensor(lambda_scale):
-        if lambda_scale.numel() != 1:
-            raise ValueError("lambda_scale must have exactly one element")
-        return lambda_scale.detach().to(device=device, dtype=dtype).reshape(1).contiguous()
+        if lambda_scale.numel() not in (1, num_heads):
+            raise ValueError("lambda_scale must have exactly one element, or one per head (%d)" % num_heads)
+        return lambda_scale.detach().to(device=device, dtype=dtype).reshape(-1).contiguous()
     return torch.tensor([float(lambda_scale)], dtype=dtype, device=device)
 
 
@@ -81,10 +83,11 @@ class _diff_attention(torch.autograd.Function):
         # k, v and upstream-gradient rows there the backward is exact on the real rows.
         n_pad = -(-N // _SEQ_MULTIPLE) * _SEQ_MULTIPLE
         q1, q2, k1, k2, v = (_pad_rows(t, n_pad) for t in (Q1, Q2, K1, K2, V))
-        lam = _lambda_tensor(LAMBDA_SCALE, dev, Q1.dtype)
+        lam = _lambda_tensor(LAMBDA_SCALE, dev, Q1.dtype, H)
         rms_norm = bool(rms_norm)
         flags = ((_FLAG_RMS_NORM if rms_norm else 0) | (_FLAG_CAUSAL if causal else 0)
-                 | (_FLAG_BF16 if Q1.dtype == torch.bfloat16 else 0))
+                 | (_FLAG_BF16 if Q1.dtype == torch.bfloat16 else 0)
+                 | (_FLAG_LAMBDA_PER_HEAD if lam.numel() > 1 else 0))
 
         y = torch.empty_like(v)
         u2 = torch.empty_like(v)
@@ -121,7 +124,7 @@ class _diff_attention(torch.autograd.Function):
         dq1, dq2 = torch.empty_like(q1), torch.empty_like(q2)
         dk1, dk2 = torch.empty_like(k1), torch.empty_like(k2)
         dv = torch.empty_like(v)
-        dlam = torch.empty(1, device=dev, dtype=q1.dtype)
+        dlam = torch.empty(lam.numel(), device=dev, dtype=q1.dtype)
         ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D)
         ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
 

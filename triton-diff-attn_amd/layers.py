@@ -24,7 +24,8 @@ def MultiheadDiffAttnKernel(
     by a per-row RMSNorm over the 2d output features and a (1 - lambda_init) scale.
 
     q1, q2, k1, k2: [B, H, N, d] fp16 on the GPU; v: [B, H, N, 2d]; lambda_scale: 1-element tensor
-    (a python float is accepted too).  Returns [B, H, N, 2d] fp16 with autograd support for the
+    (a python float is accepted too; a tensor of H elements gives every head its own lambda, which
+    the reference does not have).  Returns [B, H, N, 2d] fp16 with autograd support for the
     five tensors and lambda_scale.  `causal` (not in the reference, which lists masking as missing,
     src/kernel.py:4) lets query i attend to keys 0..i only.
     """

@@ -7,7 +7,8 @@ and (1 - lambda_init) scale, a learnable per-feature gain on the normalised head
 projection.  Attention is bidirectional unless `causal=True`.
 
   x [B, N, E]  ->  q, k [B, 2H, N, d],  v [B, H, N, 2d]      (E = 2 * H * d)
-  lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + lambda_init       (one scalar per layer)
+  lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + lambda_init       (one scalar per layer, or one per
+                                                                head with per_head_lambda=True)
   heads  = gain * MultiheadDiffAttnKernel(q1, q2, k1, k2, v, lambda, lambda_init, rms_norm=True)
   y      = out_proj(concat heads)
 """
@@ -26,7 +27,7 @@ def lambda_init_for_depth(depth: int) -> float:
 
 class DiffAttn(nn.Module):
     def __init__(self, embed_dim: int, num_heads: int, depth: int = 0, attention=MultiheadDiffAttnKernel,
-                 causal: bool = False, device=None, dtype=torch.float16):
+                 causal: bool = False, per_head_lambda: bool = False, device=None, dtype=torch.float16):
         super().__init__()
         if embed_dim % (2 * num_heads) != 0:
             raise ValueError("embed_dim must be divisible by 2 * num_heads")
@@ -43,16 +44,17 @@ class DiffAttn(nn.Module):
         self.out_proj = nn.Linear(embed_dim, embed_dim, bias=False, **kw)
         # the four lambda vectors live in fp32: their products go through exp()
         lam = dict(device=device, dtype=torch.float32)
-        self.lambda_q1 = nn.Parameter(torch.empty(self.head_dim, **lam).normal_(0.0, 0.1))
-        self.lambda_k1 = nn.Parameter(torch.empty(self.head_dim, **lam).normal_(0.0, 0.1))
-        self.lambda_q2 = nn.Parameter(torch.empty(self.head_dim, **lam).normal_(0.0, 0.1))
-        self.lambda_k2 = nn.Parameter(torch.empty(self.head_dim, **lam).normal_(0.0, 0.1))
+        shape = (num_heads, self.head_dim) if per_head_lambda else (self.head_dim,)
+        self.lambda_q1 = nn.Parameter(torch.empty(shape, **lam).normal_(0.0, 0.1))
+        self.lambda_k1 = nn.Parameter(torch.empty(shape, **lam).normal_(0.0, 0.1))
+        self.lambda_q2 = nn.Parameter(torch.empty(shape, **lam).normal_(0.0, 0.1))
+        self.lambda_k2 = nn.Parameter(torch.empty(shape, **lam).normal_(0.0, 0.1))
         self.head_gain = nn.Parameter(torch.ones(2 * self.head_dim, **kw))
 
     def lambda_scale(self) -> torch.Tensor:
-        lam = (torch.exp(torch.dot(self.lambda_q1, self.lambda_k1))
-               - torch.exp(torch.dot(self.lambda_q2, self.lambda_k2)) + self.lambda_init)
-        return lam.reshape(1)
+        lam = (torch.exp((self.lambda_q1 * self.lambda_k1).sum(-1))
+               - torch.exp((self.lambda_q2 * self.lambda_k2).sum(-1)) + self.lambda_init)
+        return lam.reshape(-1)      # [1], or [num_heads] with per_head_lambda
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         B, N, E = x.shape
