@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_symbols():
         assert hasattr(lib, name), name
         assert name in _native.SYMBOLS, "binding table misses %s" % name
-    assert lib.diffattn_abi_version() == 3
+    assert lib.diffattn_abi_version() == 3 == _native.ABI_VERSION
 
 
 def test_argument_rejection_needs_no_gpu():

@@ -11,6 +11,8 @@ import torch  # noqa: F401  (must precede loading the library)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdiffattn.so")
 
+ABI_VERSION = 3   # the version of include/diffattn.h this binding is written against
+
 _lib = None
 
 _vp = ctypes.c_void_p
@@ -49,6 +51,10 @@ def lib():
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
+        if handle.diffattn_abi_version() != ABI_VERSION:
+            raise NativeLibraryMissing(
+                "libdiffattn.so has ABI version %d, this binding needs %d: rebuild it with `python %s`"
+                % (handle.diffattn_abi_version(), ABI_VERSION, os.path.join(_HERE, "build.py")))
         _lib = handle
     return _lib
 
