@@ -65,3 +65,16 @@ def test_backward_is_deterministic():
     assert torch.equal(a[0], b[0])
     for ga, gb in zip(a[1], b[1]):
         assert torch.equal(ga, gb)
+
+
+def test_second_derivative_is_refused():
+    """The backward is a set of kernels without a derivative of its own: asking autograd to differentiate
+    through it must raise instead of returning zeros."""
+    from layers import MultiheadDiffAttnKernel
+    q1, q2, k1, k2, v, dy = (t.cuda() for t in make_inputs(1, 1, 128, 32, seed=9))
+    q1.requires_grad_(True)
+    lam = torch.tensor([0.5], dtype=torch.float16, device="cuda")
+    y = MultiheadDiffAttnKernel(q1, q2, k1, k2, v, lam, 0.8, True)
+    (g,) = torch.autograd.grad(y, q1, dy, create_graph=True)
+    with pytest.raises(RuntimeError):
+        g.float().sum().backward()

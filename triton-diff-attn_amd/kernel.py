@@ -7,6 +7,7 @@ hand-written HIP kernels in libdiffattn.so, reached through its C ABI; if the li
 the call raises -- there is no other path.
 """
 import torch
+from torch.autograd.function import once_differentiable
 
 import _native
 
@@ -111,6 +112,7 @@ class _diff_attention(torch.autograd.Function):
         return y if n_pad == N else y[:, :, :N].contiguous()
 
     @staticmethod
+    @once_differentiable        # the gradients are plain kernel outputs: a second derivative raises
     def backward(ctx, dO):
         q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam = ctx.saved_tensors
         B, H, N, D = q1.shape
