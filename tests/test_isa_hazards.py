@@ -43,3 +43,10 @@ def test_backward_kernels_have_no_unprotected_asm_mfma(tmp_path, variant):
     assert ("v_mfma_f32_32x32x16_bf16" if variant else "v_mfma_f32_32x32x16_f16") in text and ";;#ASMSTART" in text
     hazards = isa_scan.asm_mfma_hazards(text)
     assert hazards == [], "VALU write right before an inline-asm MFMA: %s" % hazards[:5]
+    # the build switches the packed-fp32 VALU instructions off; none may appear in the generated code
+    import re
+    packed = re.findall(r"^\s*(v_pk_(?:fma|mul|add)_f32)\b", text, re.M)
+    assert packed == [], "packed fp32 instructions in the backward kernels: %d" % len(packed)
+    # nothing spills: the kernels' register budgets are sized by hand
+    spills = re.findall(r"\.private_segment_fixed_size:\s*(\d+)", text)
+    assert spills and all(int(s) == 0 for s in spills), "a backward kernel uses scratch memory: %s" % spills
