@@ -78,3 +78,28 @@ def test_second_derivative_is_refused():
     (g,) = torch.autograd.grad(y, q1, dy, create_graph=True)
     with pytest.raises(RuntimeError):
         g.float().sum().backward()
+
+
+def test_forward_without_gradients_skips_the_backward_state():
+    """Under no_grad nothing is saved for a backward: the output is bit-identical and the peak memory of the
+    call drops by the tensors only a backward reads (u2 and the row statistics)."""
+    from layers import MultiheadDiffAttnKernel
+    B, H, N, D = 2, 8, 1024, 64
+    q1, q2, k1, k2, v, _ = (t.cuda() if t is not None else None for t in make_inputs(B, H, N, D, seed=10, with_dy=False))
+    lam = torch.tensor([0.5], dtype=torch.float16, device="cuda")
+
+    def peak(requires_grad):
+        q1.requires_grad_(requires_grad)
+        torch.cuda.synchronize(); torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        y = MultiheadDiffAttnKernel(q1, q2, k1, k2, v, lam, 0.8, True)
+        torch.cuda.synchronize()
+        used = torch.cuda.max_memory_allocated() - base
+        return y.detach().clone(), used
+
+    y_grad, mem_grad = peak(True)
+    y_plain, mem_plain = peak(False)
+    assert torch.equal(y_grad, y_plain)
+    v_bytes = v.numel() * 2
+    assert mem_plain <= v_bytes + (1 << 20)              # the output only
+    assert mem_grad >= 2 * v_bytes                       # output + u2 (+ statistics)

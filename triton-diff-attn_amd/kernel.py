@@ -91,19 +91,23 @@ class _diff_attention(torch.autograd.Function):
                  | (_FLAG_LAMBDA_PER_HEAD if lam.numel() > 1 else 0))
 
         y = torch.empty_like(v)
-        u2 = torch.empty_like(v)
-        lse1 = torch.empty((B, H, n_pad), device=dev, dtype=torch.float32)
-        lse2 = torch.empty((B, H, n_pad), device=dev, dtype=torch.float32)
-        rinv = torch.empty((B, H, n_pad), device=dev, dtype=torch.float32) if rms_norm else None
+        # what only a backward reads (src/kernel.py:505 saves its counterparts unconditionally) is neither
+        # allocated nor written when no input asks for a gradient, e.g. under torch.no_grad()
+        differentiable = any(ctx.needs_input_grad)
+        u2 = torch.empty_like(v) if differentiable else None
+        stat = lambda: torch.empty((B, H, n_pad), device=dev, dtype=torch.float32)
+        lse1, lse2 = (stat(), stat()) if differentiable else (None, None)
+        rinv = stat() if (rms_norm and differentiable) else None
 
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream().cuda_stream
             _native.check(lib.diffattn_forward_padded(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
-                lam.data_ptr(), y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv),
+                lam.data_ptr(), y.data_ptr(), _ptr(u2), _ptr(lse1), _ptr(lse2), _ptr(rinv),
                 B, H, n_pad, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, stream))
 
-        ctx.save_for_backward(q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam)
+        if differentiable:
+            ctx.save_for_backward(q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam)
         ctx.SM_SCALE = float(SM_SCALE)
         ctx.LAMBDA_INIT = float(LAMBDA_INIT)
         ctx.FLAGS = flags
