@@ -9,6 +9,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdiffattn.so")
+MFMA_RATE = os.path.join(HERE, "mfma_rate")
 SOURCES = ["fwd.hip", "bwd.hip", "api.hip"]
 KERNEL_SOURCES = ["fwd.hip", "bwd.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -45,6 +46,11 @@ def build(verbose=True):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
+    # a stand-alone diagnostic (not loaded by anything): the MFMA rate the GPU sustains by operand data
+    cmd = [HIPCC, *[f for f in FLAGS if f != "-fPIC"], os.path.join(CSRC, "mfma_rate.hip"), "-o", MFMA_RATE]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
     return LIB
 
 
