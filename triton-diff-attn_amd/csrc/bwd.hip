@@ -633,18 +633,24 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       f16v s1, s2, dp;
 #pragma unroll
       for (int r = 0; r < 16; ++r) { s1[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
+      // all fragments of the three score products are requested before the first product is issued
+      h8 ak1[NKS], ak2[NKS], av[NKV];
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
-        h8 a1 = *reinterpret_cast<const h8*>(sK1 + swz_off<D>(ksub * 32 + j, 16 * ks + 8 * g));
-        s1 = mfma32(a1, qf1[ks], s1);
-        h8 a2 = *reinterpret_cast<const h8*>(sK2 + swz_off<D>(ksub * 32 + j, 16 * ks + 8 * g));
-        s2 = mfma32(a2, qf2[ks], s2);
+        ak1[ks] = *reinterpret_cast<const h8*>(sK1 + swz_off<D>(ksub * 32 + j, 16 * ks + 8 * g));
+        ak2[ks] = *reinterpret_cast<const h8*>(sK2 + swz_off<D>(ksub * 32 + j, 16 * ks + 8 * g));
       }
 #pragma unroll
-      for (int kv = 0; kv < NKV; ++kv) {
-        h8 a = *reinterpret_cast<const h8*>(sV + swz_off<DV>(ksub * 32 + j, 16 * kv + 8 * g));
-        dp = mfma32(a, xf[kv], dp);
+      for (int kv = 0; kv < NKV; ++kv)
+        av[kv] = *reinterpret_cast<const h8*>(sV + swz_off<DV>(ksub * 32 + j, 16 * kv + 8 * g));
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        s1 = mfma32(ak1[ks], qf1[ks], s1);
+        s2 = mfma32(ak2[ks], qf2[ks], s2);
       }
+#pragma unroll
+      for (int kv = 0; kv < NKV; ++kv) dp = mfma32(av[kv], xf[kv], dp);
       if (ksub == 0) VTile::template issue<0, VH>(gv + (size_t)tn * BN * DV, nb + 2 * C::K_TILE, wave, lane);
       if (ksub == BN / 32 - 1) VTile::template issue<VH, VTile::PER>(gv + (size_t)tn * BN * DV, nb + 2 * C::K_TILE, wave, lane);
       if constexpr (CAUSAL) {
@@ -658,6 +664,22 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
             if (8 * (r / 4) + (r % 4) > rel) { s1[r] = -INFINITY; s2[r] = -INFINITY; }
         }
       }
+      // The transposed K fragments of the dQ products do not depend on the element-wise work: they
+      // are requested before it and arrive while it runs.  (Left to itself the compiler requests
+      // each one right in front of its product and waits out the LDS latency eight times.)
+      h8 tk1[2][NDT], tk2[2][NDT];
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const int rbase = ksub * 32 + 16 * kk + tr_row;
+#pragma unroll
+        for (int tt = 0; tt < NDT; ++tt) {
+          tk1[kk][tt] = join(lds_read_tr(sK1 + swz_off<D>(rbase, 32 * tt + tr_col)),
+                             lds_read_tr(sK1 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
+          tk2[kk][tt] = join(lds_read_tr(sK2 + swz_off<D>(rbase, 32 * tt + tr_col)),
+                             lds_read_tr(sK2 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
       h8 b1[2], b2[2];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -668,18 +690,12 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
         b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dpc, de2));   // statistic 3 is -(lambda*delta1 + delta2)
       }
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const int rbase = ksub * 32 + 16 * kk + tr_row;
+      for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
         for (int tt = 0; tt < NDT; ++tt) {
-          h8 a1 = join(lds_read_tr(sK1 + swz_off<D>(rbase, 32 * tt + tr_col)),
-                       lds_read_tr(sK1 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
-          dq1[tt] = mfma32(a1, b1[kk], dq1[tt]);
-          h8 a2 = join(lds_read_tr(sK2 + swz_off<D>(rbase, 32 * tt + tr_col)),
-                       lds_read_tr(sK2 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
-          dq2[tt] = mfma32(a2, b2[kk], dq2[tt]);
+          dq1[tt] = mfma32(tk1[kk][tt], b1[kk], dq1[tt]);
+          dq2[tt] = mfma32(tk2[kk][tt], b2[kk], dq2[tt]);
         }
-      }
     }
 
     // tile t+1 was requested one iteration ago: only this iteration's loads may remain in flight
