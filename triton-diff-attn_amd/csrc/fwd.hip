@@ -257,7 +257,9 @@ void fwd_kernel(FwdParams p) {
     load_k2(tk, kb0);
     scores(ka, s_nxt);
 
-    h8 pb[QS][NKK];      // P^T as B operands: pb[kk] covers keys 16kk..16kk+15 (accumulator order)
+    // P^T as B operands: pb[kk] covers keys 16kk..16kk+15 (accumulator order).  Built from the packed
+    // pairs as 32-bit words, so that each pair is converted once, for the row sum and the operand alike.
+    u32x4 pw[QS][NKK];
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
       float rs = 0.f;
@@ -269,8 +271,7 @@ void fwd_kernel(FwdParams p) {
           e2[0] = (half_t)fast_exp2(s_cur[qs][kt][r]);
           e2[1] = (half_t)fast_exp2(s_cur[qs][kt][r + 1]);
           rs = add_pair(e2, rs);   // row sum of the rounded probabilities
-          pb[qs][kt * 2 + r / 8][r % 8] = e2[0];
-          pb[qs][kt * 2 + r / 8][r % 8 + 1] = e2[1];
+          pw[qs][kt * 2 + r / 8][(r % 8) / 2] = __builtin_bit_cast(unsigned, e2);
         }
       l[qs] += rs;
     }
@@ -285,7 +286,7 @@ void fwd_kernel(FwdParams p) {
         h8 a = join(lds_read_tr(sV + swz_off<DV>(16 * kk + tr_row, 32 * tt + tr_col)),
                     lds_read_tr(sV + swz_off<DV>(16 * kk + 8 + tr_row, 32 * tt + tr_col)));
 #pragma unroll
-        for (int qs = 0; qs < QS; ++qs) o[qs][tt] = mfma32(a, pb[qs][kk], o[qs][tt]);
+        for (int qs = 0; qs < QS; ++qs) o[qs][tt] = mfma32(a, __builtin_bit_cast(h8, pw[qs][kk]), o[qs][tt]);
       }
     }
 
