@@ -1,0 +1,59 @@
+"""Seeded random problems: sizes, head dims and every option of the operator drawn together, so that
+combinations no hand-written case lists (a padded, causal, per-head-lambda bf16 call, say) are
+exercised against the oracle as well."""
+import random
+
+import pytest
+import torch
+
+from oracle import diff_attn_oracle as orc
+from util import GRAD_RTOL, Y_ATOL, max_abs, rel_to_max
+
+pytestmark = pytest.mark.gpu
+
+
+def draw(seed):
+    rnd = random.Random(seed)
+    return dict(
+        B=rnd.randint(1, 3), H=rnd.randint(1, 5), D=rnd.choice([32, 64, 128]),
+        N=rnd.choice([rnd.randint(1, 127), rnd.randint(129, 700), 128 * rnd.randint(1, 6)]),
+        rms=rnd.random() < 0.5, causal=rnd.random() < 0.5, per_head=rnd.random() < 0.5,
+        bf16=rnd.random() < 0.3, lambda_init=rnd.choice([0.2, 0.5, 0.8]), seed=seed)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_problem_matches_oracle(seed):
+    from layers import MultiheadDiffAttnKernel
+
+    cfg = draw(seed)
+    print("case", cfg, flush=True)
+    B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
+    dt = torch.bfloat16 if cfg["bf16"] else torch.float16
+    g = torch.Generator().manual_seed(1000 + seed)
+    mk = lambda d: torch.randn(B, H, N, d, generator=g).to(dt)
+    q1, q2, k1, k2, v, dy = mk(D), mk(D), mk(D), mk(D), mk(2 * D), mk(2 * D)
+    n_lam = H if cfg["per_head"] else 1
+    lam = (torch.rand(n_lam, generator=g) * 1.6 - 0.6).to(dt)            # in [-0.6, 1.0)
+
+    leaves = [t.cuda().requires_grad_(True) for t in (q1, q2, k1, k2, v)]
+    lam_dev = lam.cuda().requires_grad_(True)
+    extra = {"causal": True} if cfg["causal"] else {}
+    y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam_dev, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"], **extra)
+    y.backward(dy.cuda())
+    torch.cuda.synchronize()
+
+    ref = orc.forward_backward(q1, q2, k1, k2, v, lam, dy, cfg["lambda_init"], cfg["rms"], causal=cfg["causal"])
+    # bf16 carries three bits less than fp16: the tolerances of the bf16 tests
+    y_tol, g_tol = (6e-2, 8e-2) if cfg["bf16"] else (Y_ATOL, GRAD_RTOL)
+    assert y.shape == (B, H, N, 2 * D) and y.dtype == dt
+    assert max_abs(y.detach(), ref[0]) <= y_tol
+    for name, t, want in zip(("dq1", "dq2", "dk1", "dk2", "dv"), leaves, ref[1:6]):
+        scale = want.abs().max().item()
+        if scale == 0.0:
+            assert t.grad.float().abs().max().item() <= 1e-3, name      # e.g. N = 1: nothing to attend away from
+        else:
+            assert rel_to_max(t.grad, want) <= g_tol, name
+    assert lam_dev.grad.shape == (n_lam,)
+    # d(lambda) sums many terms of either sign; its error is measured against the gradient scale of the run
+    denom = max(ref[6].abs().max().item(), 1e-3 * sum(r.abs().max().item() for r in ref[1:6]) * N ** 0.5)
+    assert (lam_dev.grad.float().cpu() - ref[6]).abs().max().item() <= (3 * g_tol) * denom
