@@ -116,6 +116,8 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
  *   DIFFATTN_STAGE_DKDV    dK1, dK2, dV   (reads the workspace written by PREP)
  *   DIFFATTN_STAGE_DQ      dQ1, dQ2       (reads the workspace written by PREP)
  * diffattn_backward(...) == diffattn_backward_stages(..., DIFFATTN_STAGE_ALL, stream).
+ * The outputs of a stage that is not requested may be NULL: a caller that needs, say, only dQ1 and
+ * dQ2 passes PREP | DQ and NULL for dk1, dk2, dv and dlambda.
  */
 #define DIFFATTN_STAGE_PREP 1u
 #define DIFFATTN_STAGE_DLAMBDA 2u

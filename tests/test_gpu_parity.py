@@ -103,3 +103,24 @@ def test_forward_without_gradients_skips_the_backward_state():
     v_bytes = v.numel() * 2
     assert mem_plain <= v_bytes + (1 << 20)              # the output only
     assert mem_grad >= 2 * v_bytes                       # output + u2 (+ statistics)
+
+
+def test_only_the_requested_gradients_are_computed():
+    """With gradients asked of q1 and lambda only, the dK/dV kernel is not launched: the other inputs get no
+    gradient, and the ones asked for equal those of a full backward bit for bit."""
+    from layers import MultiheadDiffAttnKernel
+    ins = [t.cuda() for t in make_inputs(2, 3, 384, 64, seed=12)]
+    dy = ins.pop()
+
+    def run(grad_of):
+        leaves = [t.clone().requires_grad_(i in grad_of) for i, t in enumerate(ins)]
+        lam = torch.tensor([0.4], dtype=torch.float16, device="cuda", requires_grad=5 in grad_of)
+        MultiheadDiffAttnKernel(*leaves, lam, 0.8, True).backward(dy)
+        return [t.grad for t in leaves] + [lam.grad]
+
+    full = run({0, 1, 2, 3, 4, 5})
+    part = run({0, 5})
+    assert torch.equal(part[0], full[0]) and torch.equal(part[5], full[5])
+    assert all(g is None for g in part[1:5])
+    kv = run({3})
+    assert torch.equal(kv[3], full[3]) and all(g is None for i, g in enumerate(kv) if i != 3)

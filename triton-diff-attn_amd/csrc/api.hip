@@ -144,9 +144,12 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              void* workspace, size_t workspace_bytes,
                              int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                              unsigned stage_mask, void* stream) {
-  if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy ||
-      !dq1 || !dq2 || !dk1 || !dk2 || !dv || !dlambda || !workspace)
+  if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy || !workspace)
     return DIFFATTN_EINVAL_NULL;
+  // outputs are required by the stages that write them
+  if ((stage_mask & DIFFATTN_STAGE_DLAMBDA) && !dlambda) return DIFFATTN_EINVAL_NULL;
+  if ((stage_mask & DIFFATTN_STAGE_DKDV) && (!dk1 || !dk2 || !dv)) return DIFFATTN_EINVAL_NULL;
+  if ((stage_mask & DIFFATTN_STAGE_DQ) && (!dq1 || !dq2)) return DIFFATTN_EINVAL_NULL;
   if (flags & ~kKnownFlags) return DIFFATTN_EINVAL_FLAGS;
   if ((flags & DIFFATTN_RMS_NORM) && !rinv) return DIFFATTN_EINVAL_NULL;
   if (int e = check_dims(B, H, N, D)) return e;

@@ -127,26 +127,32 @@ class _diff_attention(torch.autograd.Function):
         dO = _pad_rows(dO, N)           # N is the padded length here
         n_valid = ctx.N_VALID
 
-        dq1, dq2 = torch.empty_like(q1), torch.empty_like(q2)
-        dk1, dk2 = torch.empty_like(k1), torch.empty_like(k2)
-        dv = torch.empty_like(v)
-        dlam = torch.empty(lam.numel(), device=dev, dtype=q1.dtype)
+        # only the kernels whose outputs some input asked for are launched (stage bits of the C ABI:
+        # 1 row preprocess, 2 d(lambda) reduction, 4 dK/dV, 8 dQ)
+        need = ctx.needs_input_grad
+        want_q, want_kv = need[0] or need[1], need[2] or need[3] or need[4]
+        want_lam = ctx.lambda_meta is not None and need[6]
+        stages = 1 | (2 if want_lam else 0) | (4 if want_kv else 0) | (8 if want_q else 0)
+        dq1, dq2 = (torch.empty_like(q1), torch.empty_like(q2)) if want_q else (None, None)
+        dk1, dk2, dv = (torch.empty_like(k1), torch.empty_like(k2), torch.empty_like(v)) if want_kv else (None,) * 3
+        dlam = torch.empty(lam.numel(), device=dev, dtype=q1.dtype) if want_lam else None
         ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D)
         ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
 
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream().cuda_stream
-            _native.check(lib.diffattn_backward(
+            _native.check(lib.diffattn_backward_stages(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv), dO.data_ptr(),
-                dq1.data_ptr(), dq2.data_ptr(), dk1.data_ptr(), dk2.data_ptr(), dv.data_ptr(), dlam.data_ptr(),
-                ws.data_ptr(), ws_bytes, B, H, N, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stream))
+                _ptr(dq1), _ptr(dq2), _ptr(dk1), _ptr(dk2), _ptr(dv), _ptr(dlam),
+                ws.data_ptr(), ws_bytes, B, H, N, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stages, stream))
 
         dlambda = None
-        if ctx.lambda_meta is not None and ctx.needs_input_grad[6]:
+        if want_lam:
             dtype, shape = ctx.lambda_meta
             dlambda = dlam.to(dtype).reshape(shape)
         if n_valid != N:
-            dq1, dq2, dk1, dk2, dv = (t[:, :, :n_valid].contiguous() for t in (dq1, dq2, dk1, dk2, dv))
+            dq1, dq2, dk1, dk2, dv = (None if t is None else t[:, :, :n_valid].contiguous()
+                                      for t in (dq1, dq2, dk1, dk2, dv))
         # one slot per forward argument: nine, or ten when `causal` was passed
         return (dq1, dq2, dk1, dk2, dv, None, dlambda) + (None,) * (len(ctx.needs_input_grad) - 7)
