@@ -1,4 +1,4 @@
-"""GPU parity at BASELINE.json's full sizes (configs 2, 3, 4).
+"""GPU parity at the full sizes of the benchmark configurations (2, 3 and 4).
 
 The CPU oracle cannot afford every (batch, head) unit at these sizes, and units are independent,
 so: the kernels run on the full problem; two units are checked against the fp32 oracle; the same

@@ -44,12 +44,12 @@ def test_odd_tile_counts(D, N):
 
 
 def test_config0_forward():
-    # BASELINE config 0: B=2 H=16 N=512 D=32, lambda 0.5, lambda_init 0.8, rms_norm on, forward only
+    # benchmark configuration 0: B=2 H=16 N=512 D=32, lambda 0.5, lambda_init 0.8, rms_norm on, forward only
     check_case(2, 16, 512, 32, seed=0, lam=0.5, lambda_init=0.8, rms=True, backward=False)
 
 
 def test_config1_forward_backward():
-    # BASELINE config 1: same shape and inputs as config 0, forward + backward
+    # benchmark configuration 1: same shape and inputs as config 0, forward + backward
     check_case(2, 16, 512, 32, seed=0, lam=0.5, lambda_init=0.8, rms=True, backward=True)
 
 
