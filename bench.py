@@ -161,11 +161,11 @@ def main():
         rinv = torch.empty(B, H, N, device=dev)
         grads = [torch.empty_like(t) for t in (q1, q2, k1, k2, v)]
         dlam = torch.empty(1, dtype=torch.float16, device=dev)
-        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D)
+        flags = int(cfg["rms"]) | (2 if cfg.get("causal") else 0)     # DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL
+        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D, flags)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream().cuda_stream
         sm = 1 / math.sqrt(D)
-        flags = int(cfg["rms"]) | (2 if cfg.get("causal") else 0)     # DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL
 
         def fwd_only():
             _native.check(lib.diffattn_forward(
@@ -178,7 +178,7 @@ def main():
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(), dy.data_ptr(),
                 *[g.data_ptr() for g in grads], dlam.data_ptr(), ws.data_ptr(), ws_bytes,
-                B, H, N, D, sm, cfg["lambda_init"], flags, mask, stream))
+                B, H, N, N, D, sm, cfg["lambda_init"], flags, mask, stream))
 
         fwd_only(); bwd_stage(15)()
         k_iters = max(5, min(args.steps, 30))

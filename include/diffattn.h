@@ -76,17 +76,20 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
  * Forward for a sequence whose real length n_valid is not a multiple of 128.  No counterpart in the
  * reference, whose kernels require such a multiple (src/kernel.py:4, :527).  The caller pads every
  * tensor with zero rows to N (a multiple of 128, n_valid <= N); keys n_valid..N-1 are ignored, rows
- * n_valid..N-1 of the outputs are to be discarded.  The backward needs no variant: with zero rows of
- * k1, k2, v and dy in the padding, diffattn_backward on the padded tensors returns the exact
- * gradients in rows 0..n_valid-1.  diffattn_forward is this function with n_valid = N.
+ * n_valid..N-1 of the outputs are to be discarded.  The matching backward is
+ * diffattn_backward_stages with the same n_valid, on the padded tensors with zero rows of dy in the
+ * padding; it returns the gradients of rows 0..n_valid-1.  diffattn_forward is this function with
+ * n_valid = N.
  */
 int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
                             const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
                             int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
                             void* stream);
 
-/* Bytes of device workspace diffattn_backward needs for this problem size (0 on bad sizes). */
-size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D);
+/* Bytes of device workspace diffattn_backward needs for this problem size and these flags (0 on bad
+ * sizes or unknown flag bits).  Counterpart of the scratch tensors the reference's backward
+ * allocates itself (src/kernel.py:520-529). */
+size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D, int flags);
 
 /*
  * Backward.  Replaces the launch of diff_attn_bwd (src/kernel.py:531-570) and the host-side
@@ -96,7 +99,7 @@ size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D);
  *   outputs: dq1,dq2,dk1,dk2 [B,H,N,D], dv [B,H,N,2D] fp16; dlambda: one fp16 value (H values
  *            with DIFFATTN_LAMBDA_PER_HEAD), DEVICE memory, written (not accumulated), reduced in
  *            a fixed order: bit-reproducible.
- *   workspace: device memory of at least diffattn_backward_workspace_bytes(B,H,N,D) bytes,
+ *   workspace: device memory of at least diffattn_backward_workspace_bytes(B,H,N,D,flags) bytes,
  *            256-byte aligned, contents undefined before and after.
  */
 int diffattn_backward(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
@@ -118,6 +121,8 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
  * diffattn_backward(...) == diffattn_backward_stages(..., DIFFATTN_STAGE_ALL, stream).
  * The outputs of a stage that is not requested may be NULL: a caller that needs, say, only dQ1 and
  * dQ2 passes PREP | DQ and NULL for dk1, dk2, dv and dlambda.
+ * n_valid (1..N) is the real sequence length of a problem that went through
+ * diffattn_forward_padded (N when there is no padding): keys n_valid..N-1 are ignored.
  */
 #define DIFFATTN_STAGE_PREP 1u
 #define DIFFATTN_STAGE_DLAMBDA 2u
@@ -129,7 +134,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              const float* lse1, const float* lse2, const float* rinv, const void* dy,
                              void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                              void* workspace, size_t workspace_bytes,
-                             int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
+                             int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
                              unsigned stage_mask, void* stream);
 
 #ifdef __cplusplus

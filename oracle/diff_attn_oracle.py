@@ -50,6 +50,14 @@ def _lambda_of_units(lam_values, units, H):
     return lam_values[units % H].reshape(-1, 1, 1)
 
 
+def normalise(x, lambda_init):
+    """The rms_norm branch of src/layers.py:74-78 on pre-norm rows x [..., 2D]: apex's affine-free
+    RMSNorm over the last dim (eps inside the root), then the (1 - lambda_init) factor.
+    Returns (y, rinv) with rinv [..., 1]."""
+    rinv = torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + EPS)
+    return (1 - lambda_init) * (x * rinv), rinv
+
+
 def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False, causal=False):
     """One or more (b, h) units: tensors [..., N, D] / [..., N, 2D], already in the work dtype.
 
@@ -71,8 +79,7 @@ def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False, 
     p = p1 - lam * p2                                        # src/layers.py:70
     x = torch.matmul(p, v)                                   # src/layers.py:72
     if rms_norm:                                             # src/layers.py:74-78
-        rinv = torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + EPS)
-        y = (1 - lambda_init) * (x * rinv)
+        y, rinv = normalise(x, lambda_init)
     else:
         rinv = None
         y = x

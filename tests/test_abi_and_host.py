@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_symbols():
         assert hasattr(lib, name), name
         assert name in _native.SYMBOLS, "binding table misses %s" % name
-    assert lib.diffattn_abi_version() == 3 == _native.ABI_VERSION
+    assert lib.diffattn_abi_version() == 4 == _native.ABI_VERSION
 
 
 def test_argument_rejection_needs_no_gpu():
@@ -48,20 +48,24 @@ def test_argument_rejection_needs_no_gpu():
     bad[0] = p + 2
     assert lib.diffattn_forward(*bad) == -5
     bad = args(1, 1, 128, 64)
-    bad[-2] = 16                                  # unknown flag bit
+    bad[-2] = 1 << 12                             # unknown flag bit
     assert lib.diffattn_forward(*bad) == -6
     padded = lambda n_valid: [p] * 11 + [1, 1, 128, n_valid, 64, 0.125, 0.8, 1, None]
     assert lib.diffattn_forward_padded(*padded(0)) == -3
     assert lib.diffattn_forward_padded(*padded(129)) == -3
-    assert lib.diffattn_backward_workspace_bytes(1, 1, 100, 64) == 0
-    assert lib.diffattn_backward_workspace_bytes(1, 1, 128, 48) == 0
-    need = lib.diffattn_backward_workspace_bytes(2, 3, 256, 64)
+    assert lib.diffattn_backward_workspace_bytes(1, 1, 100, 64, 0) == 0
+    assert lib.diffattn_backward_workspace_bytes(1, 1, 128, 48, 0) == 0
+    assert lib.diffattn_backward_workspace_bytes(1, 1, 128, 64, 1 << 12) == 0     # unknown flag bit
+    need = lib.diffattn_backward_workspace_bytes(2, 3, 256, 64, 1)
     rows = 2 * 3 * 256
     assert need >= rows * 128 * 2 + 4 * rows * 4
     bargs = [p] * 5 + [p, p, p, p, p, p, p] + [p] * 6 + [p, need - 1, 2, 3, 256, 64, 0.125, 0.8, 1, None]
     assert lib.diffattn_backward(*bargs) == -4
-    bargs[19], bargs[-2] = need, 32
+    bargs[19], bargs[-2] = need, 1 << 12
     assert lib.diffattn_backward(*bargs) == -6
+    sargs = lambda n_valid: bargs[:23] + [n_valid, 64, 0.125, 0.8, 1, 15, None]
+    assert lib.diffattn_backward_stages(*sargs(0)) == -3
+    assert lib.diffattn_backward_stages(*sargs(257)) == -3
     for code in (0, -1, -2, -3, -4, -5, -6):
         assert len(lib.diffattn_strerror(code)) > 0
 

@@ -58,6 +58,13 @@ def test_negative_and_zero_lambda():
     check_case(1, 2, 256, 64, seed=6, lam=0.0, lambda_init=0.8, rms=False)
 
 
+def test_lambda_init_close_to_one():
+    """The backward rebuilds the pre-norm row as Y / ((1 - lambda_init) * rinv) from the 16-bit Y: with
+    lambda_init = 0.99 the stored Y is a hundred times smaller than usual."""
+    check_case(1, 2, 256, 64, seed=21, lam=0.5, lambda_init=0.99, rms=True)
+    check_case(1, 2, 128, 32, seed=22, lam=0.3, lambda_init=0.99, rms=True)
+
+
 def test_backward_is_deterministic():
     q1, q2, k1, k2, v, dy = make_inputs(2, 4, 512, 64, seed=11)
     a = run_kernel(q1, q2, k1, k2, v, 0.5, 0.8, True, dy)
@@ -81,28 +88,35 @@ def test_second_derivative_is_refused():
 
 
 def test_forward_without_gradients_skips_the_backward_state():
-    """Under no_grad nothing is saved for a backward: the output is bit-identical and the peak memory of the
-    call drops by the tensors only a backward reads (u2 and the row statistics)."""
+    """Under no_grad nothing is saved for a backward: the output is bit-identical and the call allocates
+    only the output, not the tensors only a backward reads (u2 and the row statistics).  The allocator's
+    running total of bytes handed out is compared, which frees by earlier tests' garbage cannot lower."""
+    import gc
     from layers import MultiheadDiffAttnKernel
     B, H, N, D = 2, 8, 1024, 64
     q1, q2, k1, k2, v, _ = (t.cuda() if t is not None else None for t in make_inputs(B, H, N, D, seed=10, with_dy=False))
     lam = torch.tensor([0.5], dtype=torch.float16, device="cuda")
+    handed_out = lambda: torch.cuda.memory_stats()["allocated_bytes.all.allocated"]
 
-    def peak(requires_grad):
+    def call(requires_grad):
         q1.requires_grad_(requires_grad)
-        torch.cuda.synchronize(); torch.cuda.reset_peak_memory_stats()
-        base = torch.cuda.memory_allocated()
+        gc.collect(); torch.cuda.synchronize()
+        base = handed_out()
         y = MultiheadDiffAttnKernel(q1, q2, k1, k2, v, lam, 0.8, True)
         torch.cuda.synchronize()
-        used = torch.cuda.max_memory_allocated() - base
-        return y.detach().clone(), used
+        used = handed_out() - base
+        saved = [t for t in (y.grad_fn.saved_tensors if y.grad_fn is not None else ()) if t is not None]
+        return y.detach().clone(), used, saved
 
-    y_grad, mem_grad = peak(True)
-    y_plain, mem_plain = peak(False)
+    y_grad, mem_grad, saved_grad = call(True)
+    y_plain, mem_plain, saved_plain = call(False)
     assert torch.equal(y_grad, y_plain)
     v_bytes = v.numel() * 2
     assert mem_plain <= v_bytes + (1 << 20)              # the output only
     assert mem_grad >= 2 * v_bytes                       # output + u2 (+ statistics)
+    assert not saved_plain
+    # inputs, y, u2, two logsumexps, rinv, lambda
+    assert sum(t.shape == v.shape for t in saved_grad) >= 3 and len(saved_grad) == 11
 
 
 def test_only_the_requested_gradients_are_computed():

@@ -11,7 +11,7 @@ import torch  # noqa: F401  (must precede loading the library)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdiffattn.so")
 
-ABI_VERSION = 3   # the version of include/diffattn.h this binding is written against
+ABI_VERSION = 4   # the version of include/diffattn.h this binding is written against
 
 _lib = None
 
@@ -25,12 +25,12 @@ SYMBOLS = {
                          + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
     "diffattn_forward_padded": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp] + [ctypes.c_int] * 5
                                 + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
-    "diffattn_backward_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 4),
+    "diffattn_backward_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 5),
     "diffattn_backward": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp, _vp] + [_vp] * 6
                           + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 4
                           + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
     "diffattn_backward_stages": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp, _vp] + [_vp] * 6
-                                 + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 4
+                                 + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 5
                                  + [ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_uint, _vp]),
 }
 

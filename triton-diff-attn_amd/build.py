@@ -9,7 +9,6 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdiffattn.so")
-MFMA_RATE = os.path.join(HERE, "mfma_rate")
 ABI_EXAMPLE = os.path.join(HERE, "abi_example")
 SOURCES = ["fwd.hip", "bwd.hip", "api.hip"]
 KERNEL_SOURCES = ["fwd.hip", "bwd.hip"]
@@ -47,11 +46,6 @@ def build(verbose=True):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    # a stand-alone diagnostic (not loaded by anything): the MFMA rate the GPU sustains by operand data
-    cmd = [HIPCC, *[f for f in FLAGS if f != "-fPIC"], os.path.join(CSRC, "mfma_rate.hip"), "-o", MFMA_RATE]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
     # the C++ example of the C ABI (also driven by a GPU test): links the library, no PyTorch
     cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", os.path.join(CSRC, "abi_example.cpp"),
            "-L" + HERE, "-ldiffattn", "-Wl,-rpath,$ORIGIN", "-o", ABI_EXAMPLE]

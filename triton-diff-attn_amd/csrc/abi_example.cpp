@@ -63,7 +63,7 @@ int main(int argc, char** argv) {
   const size_t out_elems[6] = {qk, qk, qk, qk, vv, n_lambda};
   void* grad[6];
   for (int i = 0; i < 6; ++i) HIP_OK(hipMalloc(&grad[i], out_elems[i] * 2));
-  const size_t ws_bytes = diffattn_backward_workspace_bytes(B, H, N, D);
+  const size_t ws_bytes = diffattn_backward_workspace_bytes(B, H, N, D, flags);
   if (ws_bytes == 0) { fprintf(stderr, "sizes rejected\n"); return 3; }
   void* ws;
   HIP_OK(hipMalloc(&ws, ws_bytes));      // hipMalloc returns 256-byte aligned memory

@@ -67,7 +67,7 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
               const float* lse1, const float* lse2, const float* rinv, const void* dy,
               void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
               void* ws_dx, void* ws_stat, void* ws_part, int n_part,
-              int BH, int H, int N, float sm_scale, float lambda_init, int flags, unsigned stage_mask) {
+              int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags, unsigned stage_mask) {
   p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
   p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
   p.y = (const T*)y; p.u2 = (const T*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
@@ -78,6 +78,7 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
   p.BH = BH; p.N = N; p.sm_scale = sm_scale; p.lambda_init = lambda_init;
   p.rms_norm = (flags & DIFFATTN_RMS_NORM) ? 1 : 0;
   p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
+  p.n_keys = n_valid;
   p.stages = stage_mask & DIFFATTN_STAGE_ALL;
   p.H = H; p.lambda_stride = (flags & DIFFATTN_LAMBDA_PER_HEAD) ? 1 : 0;
 }
@@ -86,7 +87,7 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
 
 extern "C" {
 
-int diffattn_abi_version(void) { return 3; }
+int diffattn_abi_version(void) { return 4; }
 
 const char* diffattn_strerror(int code) {
   switch (code) {
@@ -132,8 +133,8 @@ int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, cons
   return (int)launch_fwd(p, D, (hipStream_t)stream);
 }
 
-size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D) {
-  if (check_dims(B, H, N, D)) return 0;
+size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D, int flags) {
+  if (check_dims(B, H, N, D) || (flags & ~kKnownFlags)) return 0;
   return ws_layout(B * H, N, D).total;
 }
 
@@ -142,7 +143,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              const float* lse1, const float* lse2, const float* rinv, const void* dy,
                              void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                              void* workspace, size_t workspace_bytes,
-                             int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
+                             int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
                              unsigned stage_mask, void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy || !workspace)
     return DIFFATTN_EINVAL_NULL;
@@ -153,6 +154,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   if (flags & ~kKnownFlags) return DIFFATTN_EINVAL_FLAGS;
   if ((flags & DIFFATTN_RMS_NORM) && !rinv) return DIFFATTN_EINVAL_NULL;
   if (int e = check_dims(B, H, N, D)) return e;
+  if (n_valid < 1 || n_valid > N) return DIFFATTN_EINVAL_SEQ;
   const void* ptrs[] = {q1, q2, k1, k2, v, y, u2, dy, dq1, dq2, dk1, dk2, dv};
   for (const void* q : ptrs)
     if (!aligned16(q)) return DIFFATTN_EINVAL_ALIGN;
@@ -163,12 +165,12 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   if (flags & DIFFATTN_BF16) {
     da_bf16::BwdParams p;
     fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
-             ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, sm_scale, lambda_init, flags, stage_mask);
+             ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask);
     return (int)da_bf16::launch_bwd(p, D, (hipStream_t)stream);
   }
   BwdParams p;
   fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
-           ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, sm_scale, lambda_init, flags, stage_mask);
+           ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask);
   return (int)launch_bwd(p, D, (hipStream_t)stream);
 }
 
@@ -181,7 +183,7 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
                       void* stream) {
   return diffattn_backward_stages(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy,
                                   dq1, dq2, dk1, dk2, dv, dlambda, workspace, workspace_bytes,
-                                  B, H, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, stream);
+                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, stream);
 }
 
 }  // extern "C"

@@ -537,9 +537,13 @@ struct DqCfg {
 // dQ_t = s * dS_t K_t for one block of query rows.  Every product is formed transposed,
 // [keys x queries], so that a lane owns one query column: the row statistics are per-lane
 // scalars and dS^T in accumulator layout is directly the B operand of dQ^T = K^T dS^T.
-template <int D, int NWAVES, bool CAUSAL>
+// MASK: 0 none; 1 causal (key <= query); 2 the last keys of the sequence are padding (key < n_keys).
+// A padded key has a zero K row, but its recomputed "probability" exp(0 - lse) is not small when a
+// row's logsumexp is negative, and its dS can overflow fp16: it must be masked, not multiplied by 0.
+template <int D, int NWAVES, int MASK>
 __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_waves_per_eu(DqCfg<D, NWAVES>::OCC, DqCfg<D, NWAVES>::OCC))) void bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<D, NWAVES>;
+  constexpr bool CAUSAL = (MASK == 1), PADDED = (MASK == 2);
   constexpr int DV = C::DV, NW = C::NW, BM = C::BM, BN = C::BN;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
 
@@ -599,7 +603,8 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   const half_t* gk2 = p.k2 + row0 * D;
   const half_t* gv = p.v + row0 * DV;
   // causal: keys beyond the last row of the workgroup are never visited
-  const int n_tiles = CAUSAL ? (qt + 1) * (BM / BN) : p.N / BN;
+  // padding: tiles that hold no real key are not visited either
+  const int n_tiles = CAUSAL ? (qt + 1) * (BM / BN) : PADDED ? (p.n_keys + BN - 1) / BN : p.N / BN;
   constexpr int VH = (VTile::PER + 1) / 2;
 
   const int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
@@ -659,6 +664,16 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
         const int kbase = t * BN + ksub * 32;
         if (kbase + 31 > wrow0) {
           const int rel = wrow0 + j - kbase - 4 * g;     // query index minus the key index of register 0
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (8 * (r / 4) + (r % 4) > rel) { s1[r] = -INFINITY; s2[r] = -INFINITY; }
+        }
+      }
+      if constexpr (PADDED) {
+        // only the last sub-tiles hold padding keys
+        const int kbase = t * BN + ksub * 32;
+        if (kbase + 32 > p.n_keys) {
+          const int rel = p.n_keys - 1 - kbase - 4 * g;   // last real key minus the key index of register 0
 #pragma unroll
           for (int r = 0; r < 16; ++r)
             if (8 * (r / 4) + (r % 4) > rel) { s1[r] = -INFINITY; s2[r] = -INFINITY; }
@@ -767,13 +782,17 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
     if constexpr (D != 128) {
       if (p.N % 256 == 0 && (long long)p.BH * (p.N / 128) > kNumCU) {
         wide = true;
-        if (p.causal) hipLaunchKernelGGL((bwd_dq_kernel<D, 8, true>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
-        else          hipLaunchKernelGGL((bwd_dq_kernel<D, 8, false>), dim3(p.BH * (p.N / 256)), dim3(512), 0, stream, p);
+        const dim3 grid(p.BH * (p.N / 256)), block(512);
+        if (p.causal)            hipLaunchKernelGGL((bwd_dq_kernel<D, 8, 1>), grid, block, 0, stream, p);
+        else if (p.n_keys < p.N) hipLaunchKernelGGL((bwd_dq_kernel<D, 8, 2>), grid, block, 0, stream, p);
+        else                     hipLaunchKernelGGL((bwd_dq_kernel<D, 8, 0>), grid, block, 0, stream, p);
       }
     }
     if (!wide) {
-      if (p.causal) hipLaunchKernelGGL((bwd_dq_kernel<D, 4, true>), dim3(p.BH * (p.N / 128)), dim3(256), 0, stream, p);
-      else          hipLaunchKernelGGL((bwd_dq_kernel<D, 4, false>), dim3(p.BH * (p.N / 128)), dim3(256), 0, stream, p);
+      const dim3 grid(p.BH * (p.N / 128)), block(256);
+      if (p.causal)            hipLaunchKernelGGL((bwd_dq_kernel<D, 4, 1>), grid, block, 0, stream, p);
+      else if (p.n_keys < p.N) hipLaunchKernelGGL((bwd_dq_kernel<D, 4, 2>), grid, block, 0, stream, p);
+      else                     hipLaunchKernelGGL((bwd_dq_kernel<D, 4, 0>), grid, block, 0, stream, p);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }

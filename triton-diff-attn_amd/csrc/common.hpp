@@ -153,12 +153,14 @@ __device__ __forceinline__ int swz_off(int row, int col) {
 // registers, so the per-lane address costs no vector arithmetic).  Written as inline assembly so
 // that the compiler's wait-count insertion does not serialise later, unrelated LDS reads behind
 // it; the caller orders it with wait_async_tiles() and a barrier before the data is read.
-// M0 is written without being declared: the compiler keeps it reserved (naming it as a clobber is
-// rejected with a warning) and the kernels use nothing else that goes through M0.
+// The LDS base travels in M0, bound as an operand in that physical register, so the compiler
+// owns M0: it sets it in front of the statement and knows it is live there.  The s_nop covers the
+// wait state between a write of M0 and a direct-to-LDS load, which the compiler does not insert
+// for an instruction it cannot see.
 __device__ __forceinline__ void async_copy16(const half_t* g_base, unsigned byte_off, half_t* lds_base) {
   const unsigned lds_addr = (unsigned)(unsigned long)((DA_LDS char*)lds_base);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :: "v"(byte_off), "s"(g_base), "s"(lds_addr) : "memory");
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(byte_off), "s"(g_base), "{m0}"(lds_addr) : "memory");
 }
 
 // Asynchronous copy of a dense [ROWS x COLS] fp16 tile (row stride COLS in global memory) into a

@@ -41,6 +41,7 @@ struct BwdParamsT {
   float sm_scale, lambda_init;
   int rms_norm;
   int causal;
+  int n_keys;                   // keys n_keys..N-1 are padding (N when there is none)
   unsigned stages;              // bit 0 row preprocess, 1 d(lambda) reduce, 2 dK/dV, 3 dQ
   int H;                        // heads per batch entry: unit bh belongs to head bh % H
   int lambda_stride;            // 0: one lambda; 1: one per head

@@ -80,8 +80,8 @@ class _diff_attention(torch.autograd.Function):
         lib = _native.lib()
         dev = Q1.device
         # The kernels work on multiples of 128 rows (like the reference's, src/kernel.py:527).  Other
-        # lengths are padded with zero rows here; the forward ignores the padding keys, and with zero
-        # k, v and upstream-gradient rows there the backward is exact on the real rows.
+        # lengths are padded with zero rows here; forward and backward ignore the padding keys, and a
+        # padded query row has a zero upstream gradient, so it adds nothing to dK and dV.
         n_pad = -(-N // _SEQ_MULTIPLE) * _SEQ_MULTIPLE
         q1, q2, k1, k2, v = (_pad_rows(t, n_pad) for t in (Q1, Q2, K1, K2, V))
         lam = _lambda_tensor(LAMBDA_SCALE, dev, Q1.dtype, H)
@@ -136,7 +136,7 @@ class _diff_attention(torch.autograd.Function):
         dq1, dq2 = (torch.empty_like(q1), torch.empty_like(q2)) if want_q else (None, None)
         dk1, dk2, dv = (torch.empty_like(k1), torch.empty_like(k2), torch.empty_like(v)) if want_kv else (None,) * 3
         dlam = torch.empty(lam.numel(), device=dev, dtype=q1.dtype) if want_lam else None
-        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D)
+        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D, ctx.FLAGS)
         ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
 
         with torch.cuda.device(dev):
@@ -145,7 +145,7 @@ class _diff_attention(torch.autograd.Function):
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv), dO.data_ptr(),
                 _ptr(dq1), _ptr(dq2), _ptr(dk1), _ptr(dk2), _ptr(dv), _ptr(dlam),
-                ws.data_ptr(), ws_bytes, B, H, N, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stages, stream))
+                ws.data_ptr(), ws_bytes, B, H, N, n_valid, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stages, stream))
 
         dlambda = None
         if want_lam:
