@@ -46,10 +46,10 @@ def test_short_sequences_with_large_scores(N, rms):
     assert torch.isfinite(y).all() and max_abs(y, ref[0]) <= 3 * Y_ATOL      # |v| is three times the usual
     for name, g, r in zip(("dq1", "dq2", "dk1", "dk2", "dv", "dlambda"), grads, ref[1:]):
         assert torch.isfinite(g).all(), name
-        if r.abs().max().item() < 1e-6:
-            assert g.float().abs().max().item() <= 2e-2, name      # rounding noise of 3x larger operands
-        else:
-            assert rel_to_max(g, r) <= GRAD_RTOL, name
+        # a single key has no softmax gradient and, with rms_norm, no d(lambda): what is left is the
+        # rounding noise of operands three times the usual size
+        tol = GRAD_RTOL * r.abs().max().item() if r.abs().max().item() >= 1e-3 else 2e-2
+        assert max_abs(g, r) <= tol, name
 
 
 def test_single_token_closed_form():
