@@ -34,6 +34,7 @@ extern "C" {
 #define DIFFATTN_EINVAL_WS (-4)     /* workspace too small */
 #define DIFFATTN_EINVAL_ALIGN (-5)  /* a pointer is not 16-byte aligned */
 #define DIFFATTN_EINVAL_FLAGS (-6)  /* unknown bits in `flags` */
+#define DIFFATTN_EINVAL_SCRATCH (-7) /* problem too large for diffattn_backward_static */
 
 /* `flags` of the forward and backward entry points.  DIFFATTN_RMS_NORM is the reference's boolean
  * `rms_norm` (src/kernel.py:464): a caller that passes a C boolean there keeps working.
@@ -136,6 +137,26 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              void* workspace, size_t workspace_bytes,
                              int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
                              unsigned stage_mask, void* stream);
+
+/*
+ * Backward without a workspace argument and without any allocation.  No counterpart in the
+ * reference; it is for callers that cannot allocate device memory around the call: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same operands and results
+ * as diffattn_backward (bit for bit); the workspace is a fixed array of
+ * DIFFATTN_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process
+ * ends.  Problems whose diffattn_backward_workspace_bytes exceed it are rejected with
+ * DIFFATTN_EINVAL_SCRATCH (at D = 64 the limit is about 120 000 rows B*H*N).  The device the
+ * stream belongs to must be current.  All calls on one GPU share the array: two calls that
+ * overlap in time on the same GPU (different streams or threads) race; calls on one stream are
+ * ordered and safe.
+ */
+#define DIFFATTN_STATIC_SCRATCH_BYTES (32u << 20)
+int diffattn_backward_static(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                             const void* lambda_scale, const void* y, const void* u2,
+                             const float* lse1, const float* lse2, const float* rinv, const void* dy,
+                             void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
+                             int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
+                             void* stream);
 
 #ifdef __cplusplus
 }

@@ -20,7 +20,8 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     assert declared_symbols() == sorted([
         "diffattn_abi_version", "diffattn_strerror", "diffattn_forward", "diffattn_forward_padded",
-        "diffattn_backward_workspace_bytes", "diffattn_backward", "diffattn_backward_stages"])
+        "diffattn_backward_workspace_bytes", "diffattn_backward", "diffattn_backward_stages",
+        "diffattn_backward_static"])
 
 
 def test_library_exports_every_declared_symbol():
@@ -66,7 +67,7 @@ def test_argument_rejection_needs_no_gpu():
     sargs = lambda n_valid: bargs[:23] + [n_valid, 64, 0.125, 0.8, 1, 15, None]
     assert lib.diffattn_backward_stages(*sargs(0)) == -3
     assert lib.diffattn_backward_stages(*sargs(257)) == -3
-    for code in (0, -1, -2, -3, -4, -5, -6):
+    for code in (0, -1, -2, -3, -4, -5, -6, -7):
         assert len(lib.diffattn_strerror(code)) > 0
 
 

@@ -32,6 +32,8 @@ SYMBOLS = {
     "diffattn_backward_stages": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp, _vp] + [_vp] * 6
                                  + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 5
                                  + [ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_uint, _vp]),
+    "diffattn_backward_static": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp, _vp] + [_vp] * 6
+                                 + [ctypes.c_int] * 4 + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
 }
 
 

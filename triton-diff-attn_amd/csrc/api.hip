@@ -1,7 +1,14 @@
 // C-ABI entry points of libdiffattn (declared in include/diffattn.h): argument validation,
-// workspace carve-up and kernel launches.  Nothing here allocates, synchronises or keeps state.
+// workspace carve-up and kernel launches.  Nothing here allocates or synchronises; the only state
+// is the per-device address of the built-in scratch array of diffattn_backward_static.
+#include <atomic>
+
 #include "../../include/diffattn.h"
 #include "params.hpp"
+
+// Scratch of diffattn_backward_static: one copy per GPU, at an address that differs per GPU.  In
+// host code the name is only a handle for hipGetSymbolAddress, never a device address.
+static __device__ __align__(256) unsigned char scratch[DIFFATTN_STATIC_SCRATCH_BYTES];
 
 using namespace da;
 
@@ -27,6 +34,26 @@ int check_dims(int B, int H, int N, int D) {
   // (up to 3*B*H*N floats): keep B*H*N below 2^28 rows (a 68 GiB v tensor at D = 64)
   if ((long long)B * H * N > (1LL << 28)) return DIFFATTN_EINVAL_DIM;
   if (N % 128 != 0) return DIFFATTN_EINVAL_SEQ;
+  return DIFFATTN_OK;
+}
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return DIFFATTN_EINVAL_DIM;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // every thread finds the same address
+  }
+  *out = ptr;
   return DIFFATTN_OK;
 }
 
@@ -97,6 +124,7 @@ const char* diffattn_strerror(int code) {
     case DIFFATTN_EINVAL_SEQ: return "N must be a multiple of 128 (and 1 <= n_valid <= N)";
     case DIFFATTN_EINVAL_WS: return "workspace too small or misaligned";
     case DIFFATTN_EINVAL_ALIGN: return "tensor pointers must be 16-byte aligned";
+    case DIFFATTN_EINVAL_SCRATCH: return "problem too large for the built-in scratch of diffattn_backward_static (DIFFATTN_STATIC_SCRATCH_BYTES): use diffattn_backward with a caller workspace";
     case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL, DIFFATTN_BF16, DIFFATTN_LAMBDA_PER_HEAD)";
     default: break;
   }
@@ -183,6 +211,25 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
                       void* stream) {
   return diffattn_backward_stages(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy,
                                   dq1, dq2, dk1, dk2, dv, dlambda, workspace, workspace_bytes,
+                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, stream);
+}
+
+int diffattn_backward_static(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
+                             const void* lambda_scale, const void* y, const void* u2,
+                             const float* lse1, const float* lse2, const float* rinv, const void* dy,
+                             void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
+                             int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
+                             void* stream) {
+  if (flags & ~kKnownFlags) return DIFFATTN_EINVAL_FLAGS;
+  if (int e = check_dims(B, H, N, D)) return e;
+  const size_t need = ws_layout(B * H, N, D).total;
+  if (need > (size_t)DIFFATTN_STATIC_SCRATCH_BYTES) return DIFFATTN_EINVAL_SCRATCH;
+  void* ws = nullptr;
+  if (int e = static_scratch(&ws)) return e;
+  // every byte of the workspace that a kernel reads was written earlier in the same call: nothing
+  // has to be cleared, whatever an earlier call left behind
+  return diffattn_backward_stages(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy,
+                                  dq1, dq2, dk1, dk2, dv, dlambda, ws, need,
                                   B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, stream);
 }
 
