@@ -32,6 +32,11 @@ WORKLOADS = {
     "config4": dict(B=8, H=32, N=4096, D=128, lam=0.8, lambda_init=0.2, rms=False, seed=4, scale=1.0),
     # the headline shape with the causal mask (an addition to the reference's operator)
     "headline_causal": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0, causal=True),
+    # forward-only configurations: a step is one forward without gradients
+    "config0": dict(B=2, H=16, N=512, D=32, lam=0.5, lambda_init=0.8, rms=True, seed=0, scale=1.0, fwd_only=True),
+    "headline_fwd": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0, fwd_only=True),
+    "config3": dict(B=1, H=16, N=16384, D=64, lam=0.3, lambda_init=0.8, rms=True, seed=3, scale=0.5, fwd_only=True),
+    "config3_no_norm": dict(B=1, H=16, N=16384, D=64, lam=0.3, lambda_init=0.8, rms=False, seed=3, scale=0.5, fwd_only=True),
 }
 
 
@@ -43,17 +48,31 @@ def flops(cfg):
     return 12 * unit, 20 * unit
 
 
-def event_time(fn, iters, torch):
-    """Average milliseconds per call of fn over `iters` calls, measured with events on the current stream."""
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
+def event_time(fn, iters, torch, each=None):
+    """Average milliseconds per call of fn over `iters` calls, measured with events on the current stream.
+    With a list in `each`, an event is also recorded between calls and the per-call times are appended to it."""
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(iters + 1 if each is not None else 2)]
     torch.cuda.synchronize()
-    start.record()
-    for _ in range(iters):
+    marks[0].record()
+    for i in range(iters):
         fn()
-    stop.record()
+        if each is not None:
+            marks[i + 1].record()
+    if each is None:
+        marks[1].record()
     torch.cuda.synchronize()
-    return start.elapsed_time(stop) / iters
+    if each is not None:
+        each.extend(a.elapsed_time(b) for a, b in zip(marks[:-1], marks[1:]))
+    return marks[0].elapsed_time(marks[-1]) / iters
+
+
+def quantile(values, q):
+    """Linear-interpolation quantile of a list (what the reference's do_bench reports, src/benchmark.py:94)."""
+    v = sorted(values)
+    pos = q * (len(v) - 1)
+    lo = int(pos)
+    hi = min(lo + 1, len(v) - 1)
+    return v[lo] + (v[hi] - v[lo]) * (pos - lo)
 
 
 def gpu_max_clock_mhz(torch):
@@ -85,11 +104,14 @@ def cpu_baseline(cfg, torch, budget_s=12.0):
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
     N, D = cfg["N"], cfg["D"]
-    units = 8
+    units = 8 if N <= 4096 else 2
     q1, q2, k1, k2, v, dy = make_inputs(1, units, N, D, cfg["seed"], cfg["scale"])
     lam = torch.tensor([cfg["lam"]], dtype=torch.float16)
-    run = lambda: orc.forward_backward(q1, q2, k1, k2, v, lam, dy, cfg["lambda_init"], cfg["rms"], chunk=1,
-                                       causal=bool(cfg.get("causal")))
+    if cfg.get("fwd_only"):
+        run = lambda: orc.forward(q1, q2, k1, k2, v, lam, cfg["lambda_init"], cfg["rms"], chunk=1)
+    else:
+        run = lambda: orc.forward_backward(q1, q2, k1, k2, v, lam, dy, cfg["lambda_init"], cfg["rms"], chunk=1,
+                                           causal=bool(cfg.get("causal")))
     run()  # warm-up
     t0 = time.perf_counter()
     reps = 0
@@ -99,11 +121,13 @@ def cpu_baseline(cfg, torch, budget_s=12.0):
         if time.perf_counter() - t0 > budget_s or reps >= 200:
             break
     dt = (time.perf_counter() - t0) / reps
-    fl = float(sum(flops(dict(cfg, B=1, H=units))))
+    f_fwd, f_bwd = flops(dict(cfg, B=1, H=units))
+    fl = float(f_fwd if cfg.get("fwd_only") else f_fwd + f_bwd)
     return {
         "value": fl / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": "%d of %d (batch,head) units of the workload, fp32 oracle forward+autograd backward, %d repetitions, "
-                  "%.3f s per repetition" % (units, cfg["B"] * cfg["H"], reps, dt),
+        "sample": "%d of %d (batch,head) units of the workload, fp32 oracle %s, %d repetitions, "
+                  "%.3f s per repetition" % (units, cfg["B"] * cfg["H"],
+                                             "forward" if cfg.get("fwd_only") else "forward+autograd backward", reps, dt),
     }
 
 
@@ -132,10 +156,15 @@ def main():
     lib = _native.lib()
 
     q1, q2, k1, k2, v, dy = (t.to(dev) for t in make_inputs(B, H, N, D, cfg["seed"], cfg["scale"]))
-    leaves = [t.requires_grad_(True) for t in (q1, q2, k1, k2, v)]
-    lam = torch.tensor([cfg["lam"]], dtype=torch.float16, device=dev, requires_grad=True)
+    fwd_only = bool(cfg.get("fwd_only"))
+    leaves = [t.requires_grad_(not fwd_only) for t in (q1, q2, k1, k2, v)]
+    lam = torch.tensor([cfg["lam"]], dtype=torch.float16, device=dev, requires_grad=not fwd_only)
 
     def step():
+        if fwd_only:
+            with torch.no_grad():
+                MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"])
+            return
         for t in leaves:
             t.grad = None
         lam.grad = None
@@ -146,13 +175,15 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    per_step = []
     t0 = time.perf_counter()
-    ms_events = event_time(step, args.steps, torch)
+    ms_events = event_time(step, args.steps, torch, each=per_step)
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ms_per_step = max(ms_events, wall_ms)
 
     f_fwd, f_bwd = flops(cfg)
-    value = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
+    f_step = f_fwd if fwd_only else f_fwd + f_bwd
+    value = f_step / (ms_per_step * 1e-3) / 1e12
 
     # ---- per-kernel timings through the C ABI, events on the launch stream ----
     with torch.no_grad():
@@ -167,7 +198,7 @@ def main():
         stream = torch.cuda.current_stream().cuda_stream
         sm = 1 / math.sqrt(D)
 
-        def fwd_only():
+        def launch_forward():
             _native.check(lib.diffattn_forward(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(),
@@ -180,28 +211,32 @@ def main():
                 *[g.data_ptr() for g in grads], dlam.data_ptr(), ws.data_ptr(), ws_bytes,
                 B, H, N, N, D, sm, cfg["lambda_init"], flags, mask, stream))
 
-        fwd_only(); bwd_stage(15)()
+        launch_forward()
         k_iters = max(5, min(args.steps, 30))
-        kernels_ms = {
-            "fwd_kernel": event_time(fwd_only, k_iters, torch),
-            "bwd_prep_kernel": event_time(bwd_stage(1), k_iters, torch),
-            "bwd_dlambda_kernel": event_time(bwd_stage(2), k_iters, torch),
-            "bwd_dkdv_kernel": event_time(bwd_stage(4), k_iters, torch),
-            "bwd_dq_kernel": event_time(bwd_stage(8), k_iters, torch),
-        }
+        kernels_ms = {"fwd_kernel": event_time(launch_forward, k_iters, torch)}
+        if not fwd_only:
+            bwd_stage(15)()
+            kernels_ms.update({
+                "bwd_prep_kernel": event_time(bwd_stage(1), k_iters, torch),
+                "bwd_dlambda_kernel": event_time(bwd_stage(2), k_iters, torch),
+                "bwd_dkdv_kernel": event_time(bwd_stage(4), k_iters, torch),
+                "bwd_dq_kernel": event_time(bwd_stage(8), k_iters, torch),
+            })
     unit = f_fwd // 12
-    dkdv_flops = 16 * unit      # S1,S2 (4) + dP (4) + dV (4) + dK1,dK2 (4), times B*H*N^2*D
-    dkdv_tflops = dkdv_flops / (kernels_ms["bwd_dkdv_kernel"] * 1e-3) / 1e12
+    # the dominant kernel: dK/dV backward, S1,S2 (4) + dP (4) + dV (4) + dK1,dK2 (4), times B*H*N^2*D;
+    # in a forward-only workload the forward kernel with its 12*B*H*N^2*D
+    dom, dom_flops = ("fwd_kernel", 12 * unit) if fwd_only else ("bwd_dkdv_kernel", 16 * unit)
+    dom_tflops = dom_flops / (kernels_ms[dom] * 1e-3) / 1e12
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic_headline_B4H32N2048D64.json")
-    if args.workload == "headline" and os.path.exists(tpath):
+    tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % args.workload)
+    if os.path.exists(tpath):
         # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the file's note)
-        k = json.load(open(tpath))["kernels"]["bwd_dkdv_kernel"]
-        traffic = k["fetch_bytes"] + k["write_bytes"]
+        k = json.load(open(tpath))["kernels"].get(dom)
+        traffic = k["fetch_bytes"] + k["write_bytes"] if k else None
     roofline = {
-        "bound": "mfma", "kernel": "bwd_dkdv_kernel", "achieved": dkdv_tflops, "peak": PEAK_FP16_TFLOPS,
-        "unit": "TFLOP/s", "frac": dkdv_tflops / PEAK_FP16_TFLOPS, "traffic": traffic,
-        "flops_per_launch": dkdv_flops, "ms_per_launch": kernels_ms["bwd_dkdv_kernel"],
+        "bound": "mfma", "kernel": dom, "achieved": dom_tflops, "peak": PEAK_FP16_TFLOPS,
+        "unit": "TFLOP/s", "frac": dom_tflops / PEAK_FP16_TFLOPS, "traffic": traffic,
+        "flops_per_launch": dom_flops, "ms_per_launch": kernels_ms[dom],
     }
 
     out = {
@@ -209,19 +244,25 @@ def main():
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "%s: diff-attn fwd+bwd B%d H%d N%d D%d fp16 rms_norm=%s lambda=%.1f lambda_init=%.1f"
-                               % (args.workload, B, H, N, D, cfg["rms"], cfg["lam"], cfg["lambda_init"])
+        "config": {"workload": "%s: diff-attn %s B%d H%d N%d D%d fp16 rms_norm=%s lambda=%.1f lambda_init=%.1f"
+                               % (args.workload, "fwd" if fwd_only else "fwd+bwd", B, H, N, D, cfg["rms"], cfg["lam"],
+                                  cfg["lambda_init"])
                                + (" causal" if cfg.get("causal") else "")},
         "frac_of_fp16_mfma_peak": value / PEAK_FP16_TFLOPS,
+        # the K timed steps one by one (an event between steps): median and the 5 % / 95 % quantiles
+        "ms_per_step_median": quantile(per_step, 0.5), "ms_per_step_p5": quantile(per_step, 0.05),
+        "ms_per_step_p95": quantile(per_step, 0.95),
+        "value_at_median": f_step / (quantile(per_step, 0.5) * 1e-3) / 1e12,
         "fwd_tflops": f_fwd / (kernels_ms["fwd_kernel"] * 1e-3) / 1e12,
-        "bwd_tflops": f_bwd / (sum(kernels_ms[k] for k in kernels_ms if k.startswith("bwd")) * 1e-3) / 1e12,
+        "bwd_tflops": None if fwd_only else
+        f_bwd / (sum(kernels_ms[k] for k in kernels_ms if k.startswith("bwd")) * 1e-3) / 1e12,
         "kernels_ms": kernels_ms,
         "device": {"name": prop.name, "cus": prop.multi_processor_count,
                    "clock_mhz": gpu_max_clock_mhz(torch), "peak_fp16_tflops_used": PEAK_FP16_TFLOPS},
         "roofline": roofline,
     }
     if args.workload != "headline":
-        out["metric"] = "fwd+bwd TFLOP/s & % fp16 MFMA peak, diff-attn"
+        out["metric"] = "%s TFLOP/s & %% fp16 MFMA peak, diff-attn" % ("fwd" if fwd_only else "fwd+bwd")
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, torch)
     print(json.dumps(out), flush=True)
