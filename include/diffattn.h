@@ -35,6 +35,7 @@ extern "C" {
 #define DIFFATTN_EINVAL_ALIGN (-5)  /* a pointer is not 16-byte aligned */
 #define DIFFATTN_EINVAL_FLAGS (-6)  /* unknown bits in `flags` */
 #define DIFFATTN_EINVAL_SCRATCH (-7) /* problem too large for diffattn_backward_static */
+#define DIFFATTN_EINVAL_LAYOUT (-8)  /* a stride in diffattn_layout is negative, not a multiple of 8, or a row stride is below the row width */
 
 /* `flags` of the forward and backward entry points.  DIFFATTN_RMS_NORM is the reference's boolean
  * `rms_norm` (src/kernel.py:464): a caller that passes a C boolean there keeps working.
@@ -50,6 +51,24 @@ extern "C" {
  * the backward writes H values to dlambda, each summed over the batch.  No counterpart in the
  * reference, which has one lambda per call (src/kernel.py:138). */
 #define DIFFATTN_LAMBDA_PER_HEAD 8
+
+/*
+ * Element strides of the caller's tensors, for the entry points that take a `layout`.  The
+ * reference passes the strides of Q1 (shared by Q2, K1, K2) and of V to its kernels
+ * (src/kernel.py:487-494, :552-559) and assumes O and dO dense; here y and dy have strides of
+ * their own.  Each tensor is logically [B,H,N,C] with the last dimension contiguous; `_b`, `_h`,
+ * `_n` are the distances in elements between batch entries, heads and rows.  Every stride must be
+ * a non-negative multiple of 8 (rows start 16-byte aligned) and a row stride at least C; a
+ * [B,N,H,C] buffer viewed as [B,H,N,C] is `{N*H*C, C, H*C}`.  Everything the library writes for
+ * itself or returns as a gradient (u2, the row statistics, dq1, dq2, dk1, dk2, dv) stays dense.
+ * A NULL `layout` means every tensor is dense.
+ */
+typedef struct diffattn_layout {
+  long long qk_b, qk_h, qk_n;   /* q1, q2, k1, k2  (C = D)  */
+  long long v_b, v_h, v_n;      /* v               (C = 2D) */
+  long long y_b, y_h, y_n;      /* y               (C = 2D) */
+  long long dy_b, dy_h, dy_n;   /* dy, backward only (C = 2D); ignored by the forward */
+} diffattn_layout;
 
 /* ABI version of this header; bumped when a signature changes. */
 int diffattn_abi_version(void);
@@ -80,12 +99,12 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
  * n_valid..N-1 of the outputs are to be discarded.  The matching backward is
  * diffattn_backward_stages with the same n_valid, on the padded tensors with zero rows of dy in the
  * padding; it returns the gradients of rows 0..n_valid-1.  diffattn_forward is this function with
- * n_valid = N.
+ * n_valid = N.  `layout` gives the strides of q1, q2, k1, k2, v and y (NULL: all dense).
  */
 int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
                             const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
                             int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
-                            void* stream);
+                            const diffattn_layout* layout, void* stream);
 
 /* Bytes of device workspace diffattn_backward needs for this problem size and these flags (0 on bad
  * sizes or unknown flag bits).  Counterpart of the scratch tensors the reference's backward
@@ -124,6 +143,8 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
  * dQ2 passes PREP | DQ and NULL for dk1, dk2, dv and dlambda.
  * n_valid (1..N) is the real sequence length of a problem that went through
  * diffattn_forward_padded (N when there is no padding): keys n_valid..N-1 are ignored.
+ * `layout` gives the strides of q1, q2, k1, k2, v, y and dy (NULL: all dense); the gradients are
+ * written dense.
  */
 #define DIFFATTN_STAGE_PREP 1u
 #define DIFFATTN_STAGE_DLAMBDA 2u
@@ -136,7 +157,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                              void* workspace, size_t workspace_bytes,
                              int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
-                             unsigned stage_mask, void* stream);
+                             unsigned stage_mask, const diffattn_layout* layout, void* stream);
 
 /*
  * Backward without a workspace argument and without any allocation.  No counterpart in the

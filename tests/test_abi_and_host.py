@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_symbols():
         assert hasattr(lib, name), name
         assert name in _native.SYMBOLS, "binding table misses %s" % name
-    assert lib.diffattn_abi_version() == 4 == _native.ABI_VERSION
+    assert lib.diffattn_abi_version() == 5 == _native.ABI_VERSION
 
 
 def test_argument_rejection_needs_no_gpu():
@@ -51,7 +51,7 @@ def test_argument_rejection_needs_no_gpu():
     bad = args(1, 1, 128, 64)
     bad[-2] = 1 << 12                             # unknown flag bit
     assert lib.diffattn_forward(*bad) == -6
-    padded = lambda n_valid: [p] * 11 + [1, 1, 128, n_valid, 64, 0.125, 0.8, 1, None]
+    padded = lambda n_valid, layout=None: [p] * 11 + [1, 1, 128, n_valid, 64, 0.125, 0.8, 1, layout, None]
     assert lib.diffattn_forward_padded(*padded(0)) == -3
     assert lib.diffattn_forward_padded(*padded(129)) == -3
     assert lib.diffattn_backward_workspace_bytes(1, 1, 100, 64, 0) == 0
@@ -64,10 +64,17 @@ def test_argument_rejection_needs_no_gpu():
     assert lib.diffattn_backward(*bargs) == -4
     bargs[19], bargs[-2] = need, 1 << 12
     assert lib.diffattn_backward(*bargs) == -6
-    sargs = lambda n_valid: bargs[:23] + [n_valid, 64, 0.125, 0.8, 1, 15, None]
+    sargs = lambda n_valid, layout=None: bargs[:23] + [n_valid, 64, 0.125, 0.8, 1, 15, layout, None]
     assert lib.diffattn_backward_stages(*sargs(0)) == -3
     assert lib.diffattn_backward_stages(*sargs(257)) == -3
-    for code in (0, -1, -2, -3, -4, -5, -6, -7):
+    # strides: multiples of 8 elements, rows at least as far apart as they are wide
+    good = dict(qk_b=128 * 64, qk_h=64, qk_n=64, v_b=128 * 128, v_h=128, v_n=128,
+                y_b=128 * 128, y_h=128, y_n=128, dy_b=128 * 128, dy_h=128, dy_n=128)
+    for field, value in (("qk_n", 32), ("v_n", 132), ("y_h", -8), ("dy_b", 4)):
+        lay = _native.Layout(**dict(good, **{field: value}))
+        assert lib.diffattn_forward_padded(*padded(128, ctypes.byref(lay))) == -8, field
+        assert lib.diffattn_backward_stages(*sargs(256, ctypes.byref(lay))) == -8, field
+    for code in (0, -1, -2, -3, -4, -5, -6, -7, -8):
         assert len(lib.diffattn_strerror(code)) > 0
 
 
@@ -97,7 +104,12 @@ def test_host_validation_errors():
     padded = _pad_rows(x, 8)
     assert padded.shape == (2, 3, 8, 4) and padded.is_contiguous()
     assert torch.equal(padded[:, :, :5], x) and padded[:, :, 5:].abs().sum() == 0
-    assert _pad_rows(x, 5) is x
+    from kernel import _in_place, _is_dense, _strides_ok
+    wide = torch.zeros(2, 16, 3, 64, dtype=torch.float16)              # a [B,N,H,C] buffer seen as [B,H,N,C]
+    view = wide.transpose(1, 2)
+    assert _strides_ok(view) and _in_place(view) is view and not _is_dense(view) and _is_dense(wide)
+    assert not _strides_ok(x.transpose(2, 3)) and _in_place(x.transpose(2, 3)).is_contiguous()    # last dim strided
+    assert not _strides_ok(torch.zeros(2, 3, 5, 36, dtype=torch.float16)[..., :32])               # rows not 16-byte aligned
     lam = _lambda_tensor(0.25, torch.device("cpu"))
     assert lam.dtype == torch.float16 and lam.shape == (1,) and lam.item() == 0.25
 

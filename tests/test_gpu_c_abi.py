@@ -24,13 +24,16 @@ def as_u16(t):
     return t.contiguous().view(torch.int16).numpy().astype(np.int16).tobytes()
 
 
-@pytest.mark.parametrize("B,H,N,D,flags", [
-    (2, 3, 256, 64, RMS),
-    (1, 4, 384, 32, RMS | CAUSAL | PER_HEAD),
-    (1, 2, 128, 128, 0),
-    (2, 2, 256, 64, RMS | BF16),
+@pytest.mark.parametrize("B,H,N,D,flags,token_major", [
+    (2, 3, 256, 64, RMS, False),
+    (1, 4, 384, 32, RMS | CAUSAL | PER_HEAD, False),
+    (1, 2, 128, 128, 0, False),
+    (2, 2, 256, 64, RMS | BF16, False),
+    (2, 3, 256, 64, RMS, True),              # [B,N,H,C] buffers handed over through diffattn_layout
+    (2, 5, 384, 32, CAUSAL, True),
+    (1, 3, 128, 128, RMS, True),
 ])
-def test_cpp_program_matches_oracle(tmp_path, B, H, N, D, flags):
+def test_cpp_program_matches_oracle(tmp_path, B, H, N, D, flags, token_major):
     assert os.path.exists(EXE), "abi_example is not built: run python triton-diff-attn_amd/build.py"
     dt = torch.bfloat16 if flags & BF16 else torch.float16
     g = torch.Generator().manual_seed(77 + flags)
@@ -41,10 +44,12 @@ def test_cpp_program_matches_oracle(tmp_path, B, H, N, D, flags):
     fin, fout = tmp_path / "in.bin", tmp_path / "out.bin"
     with open(fin, "wb") as f:
         f.write(struct.pack("<5i2f", B, H, N, D, flags, lambda_init, sm_scale))
-        for t in (q1, q2, k1, k2, v, dy, lam):
-            f.write(as_u16(t))
+        for t in (q1, q2, k1, k2, v, dy):
+            f.write(as_u16(t.transpose(1, 2) if token_major else t))
+        f.write(as_u16(lam))
     print("case", B, H, N, D, flags, flush=True)
-    run = subprocess.run([EXE, str(fin), str(fout)], capture_output=True, text=True, timeout=100)
+    run = subprocess.run([EXE, str(fin), str(fout)] + (["token-major"] if token_major else []),
+                         capture_output=True, text=True, timeout=100)
     assert run.returncode == 0, run.stderr
     raw = np.fromfile(fout, dtype=np.int16)
     qk, vv = B * H * N * D, B * H * N * 2 * D
@@ -56,6 +61,7 @@ def test_cpp_program_matches_oracle(tmp_path, B, H, N, D, flags):
         pos += n
     ref = orc.forward_backward(q1, q2, k1, k2, v, lam, dy, lambda_init, bool(flags & RMS), causal=bool(flags & CAUSAL))
     y_tol, g_tol = (6e-2, 8e-2) if flags & BF16 else (Y_ATOL, GRAD_RTOL)
-    assert max_abs(outs[0].reshape(ref[0].shape), ref[0]) <= y_tol
+    y = outs[0].reshape(B, N, H, 2 * D).transpose(1, 2) if token_major else outs[0].reshape(ref[0].shape)
+    assert max_abs(y, ref[0]) <= y_tol
     for name, got, want in zip(("dq1", "dq2", "dk1", "dk2", "dv", "dlambda"), outs[1:], ref[1:]):
         assert rel_to_max(got.reshape(want.shape), want) <= g_tol, name

@@ -2,7 +2,11 @@
 // hipMalloc, a stream of its own, forward and backward of one problem read from a file.  It is the
 // example that goes with include/diffattn.h and the program tests/test_gpu_c_abi.py drives.
 //
-//   abi_example <in.bin> <out.bin>
+//   abi_example <in.bin> <out.bin> [token-major]
+//
+// With a third argument the tensors q1, q2, k1, k2, v, dy of in.bin and y of out.bin are stored
+// [B,N,H,C] (the layout a projection writes) and are handed to the library as they are, through the
+// strides of diffattn_layout; the gradients always come back dense [B,H,N,C].
 //
 // in.bin : int32 B, H, N, D, flags; float32 lambda_init, sm_scale; then the 16-bit tensors q1, q2, k1,
 //          k2 [B,H,N,D], v, dy [B,H,N,2D] and lambda (1 or H values), all in the dtype the flags name
@@ -28,7 +32,8 @@
   } while (0)
 
 int main(int argc, char** argv) {
-  if (argc != 3) { fprintf(stderr, "usage: %s in.bin out.bin\n", argv[0]); return 1; }
+  if (argc != 3 && argc != 4) { fprintf(stderr, "usage: %s in.bin out.bin [token-major]\n", argv[0]); return 1; }
+  const bool token_major = (argc == 4);
   FILE* f = fopen(argv[1], "rb");
   if (!f) { perror(argv[1]); return 1; }
   int32_t hdr[5];
@@ -68,11 +73,23 @@ int main(int argc, char** argv) {
   void* ws;
   HIP_OK(hipMalloc(&ws, ws_bytes));      // hipMalloc returns 256-byte aligned memory
 
-  DA_OK(diffattn_forward(in[0], in[1], in[2], in[3], in[4], in[6], y, u2, lse1, lse2, rinv,
-                         B, H, N, D, sm_scale, lambda_init, flags, stream));
-  DA_OK(diffattn_backward(in[0], in[1], in[2], in[3], in[4], in[6], y, u2, lse1, lse2, rinv, in[5],
-                          grad[0], grad[1], grad[2], grad[3], grad[4], grad[5], ws, ws_bytes,
-                          B, H, N, D, sm_scale, lambda_init, flags, stream));
+  if (token_major) {
+    // a [B,N,H,C] buffer seen as [B,H,N,C]: batch stride N*H*C, head stride C, row stride H*C
+    const long long d = D, dv = 2 * D;
+    const diffattn_layout lay = {(long long)N * H * d, d, H * d, (long long)N * H * dv, dv, H * dv,
+                                 (long long)N * H * dv, dv, H * dv, (long long)N * H * dv, dv, H * dv};
+    DA_OK(diffattn_forward_padded(in[0], in[1], in[2], in[3], in[4], in[6], y, u2, lse1, lse2, rinv,
+                                  B, H, N, N, D, sm_scale, lambda_init, flags, &lay, stream));
+    DA_OK(diffattn_backward_stages(in[0], in[1], in[2], in[3], in[4], in[6], y, u2, lse1, lse2, rinv, in[5],
+                                   grad[0], grad[1], grad[2], grad[3], grad[4], grad[5], ws, ws_bytes,
+                                   B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, &lay, stream));
+  } else {
+    DA_OK(diffattn_forward(in[0], in[1], in[2], in[3], in[4], in[6], y, u2, lse1, lse2, rinv,
+                           B, H, N, D, sm_scale, lambda_init, flags, stream));
+    DA_OK(diffattn_backward(in[0], in[1], in[2], in[3], in[4], in[6], y, u2, lse1, lse2, rinv, in[5],
+                            grad[0], grad[1], grad[2], grad[3], grad[4], grad[5], ws, ws_bytes,
+                            B, H, N, D, sm_scale, lambda_init, flags, stream));
+  }
   HIP_OK(hipStreamSynchronize(stream));
 
   FILE* o = fopen(argv[2], "wb");

@@ -57,6 +57,31 @@ int static_scratch(void** out) {
   return DIFFATTN_OK;
 }
 
+// Layout of the strided tensors: the caller's, or dense [B,H,N,C] when none is given.
+struct Layouts { da_abi::Strides qk, v, y, dy; };
+
+inline da_abi::Strides dense(int H, int N, int C) { return {(long long)H * N * C, (long long)N * C, (long long)C}; }
+
+inline bool stride_ok(long long b, long long h, long long n, int C) {
+  // rows are contiguous and at least C apart; every row starts on a 16-byte boundary; the kernels
+  // form 32-bit byte offsets of up to 16 rows
+  return n >= C && n % 8 == 0 && n <= (1LL << 26) && b >= 0 && h >= 0 && b % 8 == 0 && h % 8 == 0;
+}
+
+int resolve_layout(const diffattn_layout* l, int H, int N, int D, Layouts* out) {
+  out->qk = dense(H, N, D);
+  out->v = out->y = out->dy = dense(H, N, 2 * D);
+  if (!l) return DIFFATTN_OK;
+  if (!stride_ok(l->qk_b, l->qk_h, l->qk_n, D) || !stride_ok(l->v_b, l->v_h, l->v_n, 2 * D) ||
+      !stride_ok(l->y_b, l->y_h, l->y_n, 2 * D) || !stride_ok(l->dy_b, l->dy_h, l->dy_n, 2 * D))
+    return DIFFATTN_EINVAL_LAYOUT;
+  out->qk = {l->qk_b, l->qk_h, l->qk_n};
+  out->v = {l->v_b, l->v_h, l->v_n};
+  out->y = {l->y_b, l->y_h, l->y_n};
+  out->dy = {l->dy_b, l->dy_h, l->dy_n};
+  return DIFFATTN_OK;
+}
+
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 struct WsLayout {
@@ -77,7 +102,8 @@ WsLayout ws_layout(int BH, int N, int D) {
 template <class T>
 void fill_fwd(da_abi::FwdParamsT<T>& p, const void* q1, const void* q2, const void* k1, const void* k2,
               const void* v, const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
-              int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags) {
+              int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags, const Layouts& lay) {
+  p.sqk = lay.qk; p.sv = lay.v; p.sy = lay.y;
   p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
   p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
   p.y = (T*)y; p.u2 = (T*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
@@ -94,7 +120,9 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
               const float* lse1, const float* lse2, const float* rinv, const void* dy,
               void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
               void* ws_dx, void* ws_stat, void* ws_part, int n_part,
-              int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags, unsigned stage_mask) {
+              int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags, unsigned stage_mask,
+              const Layouts& lay) {
+  p.sqk = lay.qk; p.sv = lay.v; p.sy = lay.y; p.sdy = lay.dy;
   p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
   p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
   p.y = (const T*)y; p.u2 = (const T*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
@@ -114,7 +142,7 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
 
 extern "C" {
 
-int diffattn_abi_version(void) { return 4; }
+int diffattn_abi_version(void) { return 5; }
 
 const char* diffattn_strerror(int code) {
   switch (code) {
@@ -125,6 +153,7 @@ const char* diffattn_strerror(int code) {
     case DIFFATTN_EINVAL_WS: return "workspace too small or misaligned";
     case DIFFATTN_EINVAL_ALIGN: return "tensor pointers must be 16-byte aligned";
     case DIFFATTN_EINVAL_SCRATCH: return "problem too large for the built-in scratch of diffattn_backward_static (DIFFATTN_STATIC_SCRATCH_BYTES): use diffattn_backward with a caller workspace";
+    case DIFFATTN_EINVAL_LAYOUT: return "bad strides in diffattn_layout: every stride must be a non-negative multiple of 8 elements and a row stride at least the row width";
     case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL, DIFFATTN_BF16, DIFFATTN_LAMBDA_PER_HEAD)";
     default: break;
   }
@@ -137,13 +166,13 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
                      int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                      void* stream) {
   return diffattn_forward_padded(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv,
-                                 B, H, N, N, D, sm_scale, lambda_init, flags, stream);
+                                 B, H, N, N, D, sm_scale, lambda_init, flags, nullptr, stream);
 }
 
 int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
                             const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
                             int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
-                            void* stream) {
+                            const diffattn_layout* layout, void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y) return DIFFATTN_EINVAL_NULL;
   if (flags & ~kKnownFlags) return DIFFATTN_EINVAL_FLAGS;
   if (int e = check_dims(B, H, N, D)) return e;
@@ -151,13 +180,15 @@ int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, cons
   if (!aligned16(q1) || !aligned16(q2) || !aligned16(k1) || !aligned16(k2) || !aligned16(v) ||
       !aligned16(y) || !aligned16(u2))
     return DIFFATTN_EINVAL_ALIGN;
+  Layouts lay;
+  if (int e = resolve_layout(layout, H, N, D, &lay)) return e;
   if (flags & DIFFATTN_BF16) {
     da_bf16::FwdParams p;
-    fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags);
+    fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags, lay);
     return (int)da_bf16::launch_fwd(p, D, (hipStream_t)stream);
   }
   FwdParams p;
-  fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags);
+  fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags, lay);
   return (int)launch_fwd(p, D, (hipStream_t)stream);
 }
 
@@ -172,7 +203,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                              void* workspace, size_t workspace_bytes,
                              int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
-                             unsigned stage_mask, void* stream) {
+                             unsigned stage_mask, const diffattn_layout* layout, void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy || !workspace)
     return DIFFATTN_EINVAL_NULL;
   // outputs are required by the stages that write them
@@ -186,6 +217,8 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   const void* ptrs[] = {q1, q2, k1, k2, v, y, u2, dy, dq1, dq2, dk1, dk2, dv};
   for (const void* q : ptrs)
     if (!aligned16(q)) return DIFFATTN_EINVAL_ALIGN;
+  Layouts lay;
+  if (int e = resolve_layout(layout, H, N, D, &lay)) return e;
   const WsLayout w = ws_layout(B * H, N, D);
   if (workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return DIFFATTN_EINVAL_WS;
   char* ws = (char*)workspace;
@@ -193,12 +226,12 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   if (flags & DIFFATTN_BF16) {
     da_bf16::BwdParams p;
     fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
-             ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask);
+             ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask, lay);
     return (int)da_bf16::launch_bwd(p, D, (hipStream_t)stream);
   }
   BwdParams p;
   fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
-           ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask);
+           ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask, lay);
   return (int)launch_bwd(p, D, (hipStream_t)stream);
 }
 
@@ -211,7 +244,7 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
                       void* stream) {
   return diffattn_backward_stages(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy,
                                   dq1, dq2, dk1, dk2, dv, dlambda, workspace, workspace_bytes,
-                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, stream);
+                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, nullptr, stream);
 }
 
 int diffattn_backward_static(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
@@ -230,7 +263,7 @@ int diffattn_backward_static(const void* q1, const void* q2, const void* k1, con
   // has to be cleared, whatever an earlier call left behind
   return diffattn_backward_stages(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy,
                                   dq1, dq2, dk1, dk2, dv, dlambda, ws, need,
-                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, stream);
+                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, nullptr, stream);
 }
 
 }  // extern "C"

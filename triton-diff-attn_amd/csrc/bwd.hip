@@ -30,7 +30,11 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
   __shared__ float red[256];
   const int tid = threadIdx.x, sub = tid % LPR, rloc = tid / LPR;
   // the 64 rows of a workgroup belong to one (batch, head) unit: N is a multiple of 128
-  const float lam = da_abi::lambda_of_unit(p, (int)(((size_t)blockIdx.x * kPrepRows) / p.N));
+  const int bh = (int)(((size_t)blockIdx.x * kPrepRows) / p.N);
+  const int n0 = (int)(((size_t)blockIdx.x * kPrepRows) % p.N);
+  const float lam = da_abi::lambda_of_unit(p, bh);
+  const half_t* gy = p.y + da_abi::unit_base(p, p.sy, bh) + 8 * sub;
+  const half_t* gdy = p.dy + da_abi::unit_base(p, p.sdy, bh) + 8 * sub;
   const float c = 1.0f - p.lambda_init;
   const size_t rows = (size_t)p.BH * p.N;
   float part = 0.f;
@@ -38,9 +42,10 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
   for (int pass = 0; pass < kPrepRows / RPP; ++pass) {
     const size_t row = (size_t)blockIdx.x * kPrepRows + pass * RPP + rloc;
     const size_t off = row * DV + 8 * sub;
-    const h8 y8 = *reinterpret_cast<const h8*>(p.y + off);
+    const size_t n = (size_t)(n0 + pass * RPP + rloc);
+    const h8 y8 = *reinterpret_cast<const h8*>(gy + n * (size_t)p.sy.n);
     const h8 u8 = *reinterpret_cast<const h8*>(p.u2 + off);
-    const h8 g8 = *reinterpret_cast<const h8*>(p.dy + off);
+    const h8 g8 = *reinterpret_cast<const h8*>(gdy + n * (size_t)p.sdy.n);
     float dx[8], x[8];
     if (RMS) {
       float gy = 0.f;
@@ -171,6 +176,9 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   const size_t rows = (size_t)p.BH * p.N;
   const size_t row0 = (size_t)bh * p.N;
   const int key = kt * BK + wave * 32 + j;
+  // element offsets of the unit's first row and the row strides of the strided tensors
+  const size_t qk_base = da_abi::unit_base(p, p.sqk, bh), v_base = da_abi::unit_base(p, p.sv, bh);
+  const int qk_n = (int)p.sqk.n, v_n = (int)p.sv.n;
 
   const float c = p.sm_scale * kLog2e;
   const float lam = da_abi::lambda_of_unit(p, bh);
@@ -178,9 +186,9 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   // persistent B operands: this lane's key row of K1, K2, V
   h8 kf1[NKS], kf2[NKS], vf[NKV];
   {
-    const half_t* r1 = p.k1 + (row0 + key) * D + 8 * g;
-    const half_t* r2 = p.k2 + (row0 + key) * D + 8 * g;
-    const half_t* rv = p.v + (row0 + key) * DV + 8 * g;
+    const half_t* r1 = p.k1 + qk_base + (size_t)key * qk_n + 8 * g;
+    const half_t* r2 = p.k2 + qk_base + (size_t)key * qk_n + 8 * g;
+    const half_t* rv = p.v + v_base + (size_t)key * v_n + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       // pre-multiplied by sm_scale*log2(e): the score products come out in log2 units
@@ -214,9 +222,10 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
 
   using QTile = AsyncTile<BQ, D, NW>;
   using XTile = AsyncTile<BQ, DV, NW>;
-  const half_t* gq1 = p.q1 + row0 * D;
-  const half_t* gq2 = p.q2 + row0 * D;
+  const half_t* gq1 = p.q1 + qk_base;
+  const half_t* gq2 = p.q2 + qk_base;
   const half_t* gx = p.dx + row0 * DV;
+  const unsigned q_off = QTile::lane_off(wave, lane, qk_n);
   // the 4 x BQ statistics of a query tile are one piece of 16*BQ bytes: lane l < BQ fetches
   // stat[l / (BQ/4)][4 * (l % (BQ/4)) .. +3]
   const float* gstat = p.stat + row0;
@@ -226,10 +235,10 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   auto stage = [&](int qt, int buf, int part) {
     half_t* b = smem + buf * C::STAGE;
     if (part == 0) {
-      QTile::issue(gq1 + (size_t)qt * BQ * D, b, wave, lane);
+      QTile::issue_at(gq1 + (size_t)qt * BQ * qk_n, b, wave, lane, q_off, qk_n);
       if (wave == 0 && lane < BQ) async_copy16(reinterpret_cast<const half_t*>(gstat + (size_t)qt * BQ), stat_off, b + 2 * C::Q_TILE + C::X_TILE);
     } else if (part == 1) {
-      QTile::issue(gq2 + (size_t)qt * BQ * D, b + C::Q_TILE, wave, lane);
+      QTile::issue_at(gq2 + (size_t)qt * BQ * qk_n, b + C::Q_TILE, wave, lane, q_off, qk_n);
     } else if (part == 2) {
       XTile::template issue<0, XH>(gx + (size_t)qt * BQ * DV, b + 2 * C::Q_TILE, wave, lane);
     } else {
@@ -565,6 +574,9 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   const size_t rows = (size_t)p.BH * p.N;
   const size_t row0 = (size_t)bh * p.N;
   const size_t qrow = row0 + qt * BM + wave * 32 + j;
+  // element offsets of the unit's first row and the row strides of the strided tensors
+  const size_t qk_base = da_abi::unit_base(p, p.sqk, bh), v_base = da_abi::unit_base(p, p.sv, bh);
+  const int qk_n = (int)p.sqk.n, v_n = (int)p.sv.n;
 
   const float lam = da_abi::lambda_of_unit(p, bh);
 
@@ -574,8 +586,8 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   h8 qf1[NKS], qf2[NKS], xf[NKV];
   {
     const float c = p.sm_scale * kLog2e;
-    const half_t* r1 = p.q1 + qrow * D + 8 * g;
-    const half_t* r2 = p.q2 + qrow * D + 8 * g;
+    const half_t* r1 = p.q1 + qk_base + (size_t)(qt * BM + wave * 32 + j) * qk_n + 8 * g;
+    const half_t* r2 = p.q2 + qk_base + (size_t)(qt * BM + wave * 32 + j) * qk_n + 8 * g;
     const half_t* rx = p.dx + qrow * DV + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
@@ -599,9 +611,10 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
 
   using KTile = AsyncTile<BN, D, NW>;
   using VTile = AsyncTile<BN, DV, NW>;
-  const half_t* gk1 = p.k1 + row0 * D;
-  const half_t* gk2 = p.k2 + row0 * D;
-  const half_t* gv = p.v + row0 * DV;
+  const half_t* gk1 = p.k1 + qk_base;
+  const half_t* gk2 = p.k2 + qk_base;
+  const half_t* gv = p.v + v_base;
+  const unsigned k_off = KTile::lane_off(wave, lane, qk_n), v_off = VTile::lane_off(wave, lane, v_n);
   // causal: keys beyond the last row of the workgroup are never visited
   // padding: tiles that hold no real key are not visited either
   const int n_tiles = CAUSAL ? (qt + 1) * (BM / BN) : PADDED ? (p.n_keys + BN - 1) / BN : p.N / BN;
@@ -610,9 +623,9 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   const int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
   auto fetch_all = [&](int t, int buf) {
     half_t* b = smem + buf * C::STAGE;
-    KTile::issue(gk1 + (size_t)t * BN * D, b, wave, lane);
-    KTile::issue(gk2 + (size_t)t * BN * D, b + C::K_TILE, wave, lane);
-    VTile::issue(gv + (size_t)t * BN * DV, b + 2 * C::K_TILE, wave, lane);
+    KTile::issue_at(gk1 + (size_t)t * BN * qk_n, b, wave, lane, k_off, qk_n);
+    KTile::issue_at(gk2 + (size_t)t * BN * qk_n, b + C::K_TILE, wave, lane, k_off, qk_n);
+    VTile::issue_at(gv + (size_t)t * BN * v_n, b + 2 * C::K_TILE, wave, lane, v_off, v_n);
   };
   fetch_all(0, 0);
   fetch_all((n_tiles > 1) ? 1 : 0, 1);
@@ -629,11 +642,11 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
     const half_t* sV = sK1 + 2 * C::K_TILE;
     half_t* nb = smem + bnext * C::STAGE;            // held tile t-1, consumed one iteration ago
     const int tn = (t + 2 < n_tiles) ? t + 2 : n_tiles - 1;   // past the end: harmless re-reads
-    KTile::issue(gk1 + (size_t)tn * BN * D, nb, wave, lane);
+    KTile::issue_at(gk1 + (size_t)tn * BN * qk_n, nb, wave, lane, k_off, qk_n);
 
 #pragma unroll
     for (int ksub = 0; ksub < BN / 32; ++ksub) {
-      if (ksub == 0) KTile::issue(gk2 + (size_t)tn * BN * D, nb + C::K_TILE, wave, lane);
+      if (ksub == 0) KTile::issue_at(gk2 + (size_t)tn * BN * qk_n, nb + C::K_TILE, wave, lane, k_off, qk_n);
       // transposed tiles [32 keys x 32 queries]: this lane's column is its query
       f16v s1, s2, dp;
 #pragma unroll
@@ -656,8 +669,8 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       }
 #pragma unroll
       for (int kv = 0; kv < NKV; ++kv) dp = mfma32(av[kv], xf[kv], dp);
-      if (ksub == 0) VTile::template issue<0, VH>(gv + (size_t)tn * BN * DV, nb + 2 * C::K_TILE, wave, lane);
-      if (ksub == BN / 32 - 1) VTile::template issue<VH, VTile::PER>(gv + (size_t)tn * BN * DV, nb + 2 * C::K_TILE, wave, lane);
+      if (ksub == 0) VTile::template issue_at<0, VH>(gv + (size_t)tn * BN * v_n, nb + 2 * C::K_TILE, wave, lane, v_off, v_n);
+      if (ksub == BN / 32 - 1) VTile::template issue_at<VH, VTile::PER>(gv + (size_t)tn * BN * v_n, nb + 2 * C::K_TILE, wave, lane, v_off, v_n);
       if constexpr (CAUSAL) {
         // only the last sub-tiles of a wave's loop reach past its first row: mask key > query there
         const int wrow0 = qt * BM + wave * 32;

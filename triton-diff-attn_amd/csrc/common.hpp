@@ -163,27 +163,28 @@ __device__ __forceinline__ void async_copy16(const half_t* g_base, unsigned byte
                :: "v"(byte_off), "s"(g_base), "{m0}"(lds_addr) : "memory");
 }
 
-// Asynchronous copy of a dense [ROWS x COLS] fp16 tile (row stride COLS in global memory) into a
-// swizzled LDS tile with direct global->LDS loads: no registers, no LDS store instructions.  One
-// wave-instruction moves 64 chunks (1 KiB, contiguous in global memory as well); the hardware
-// writes lane l's 16 bytes at (wave-uniform LDS base) + 16*l, so the swizzle is applied by
-// choosing which global chunk of the 1 KiB piece each lane fetches.  NW waves share the tile's
-// instructions round-robin.  Completion: s_waitcnt vmcnt(0), then a barrier.
+// Asynchronous copy of a [ROWS x COLS] fp16 tile whose rows are `stride` elements apart in global
+// memory (each row contiguous) into a swizzled LDS tile with direct global->LDS loads: no
+// registers, no LDS store instructions.  One wave-instruction moves a piece of 64 chunks (1 KiB,
+// RPP whole rows); the hardware writes lane l's 16 bytes at (wave-uniform LDS base) + 16*l, so the
+// swizzle is applied by choosing which global chunk of the piece each lane fetches.  NW waves
+// share the tile's instructions round-robin.  Completion: s_waitcnt vmcnt(0), then a barrier.
 template <int ROWS, int COLS, int NW>
 struct AsyncTile {
   static constexpr int CPR = COLS / 8;
+  static constexpr int RPP = 64 / CPR;        // rows per piece
   static constexpr int NINST = ROWS * CPR / 64;
   static constexpr int PER = (NINST + NW - 1) / NW;
-  static_assert((ROWS * CPR) % 64 == 0, "tile must be a whole number of 1 KiB pieces");
+  static_assert((ROWS * CPR) % 64 == 0 && 64 % CPR == 0, "tile must be a whole number of 1 KiB pieces of whole rows");
   // The swizzle of a piece depends on the piece index only through a few low bits; when the
   // wave's pieces (wave, wave + NW, ...) agree in those bits, one per-lane offset serves them all.
   static constexpr bool kOneOffset = (CPR == 4) || (CPR == 8 && NW % 2 == 0) || (CPR == 16 && NW % 4 == 0) ||
                                      (CPR == 32 && NW % 8 == 0);
-  // byte offset inside piece `inst` of the chunk that `lane` fetches
-  __device__ static __forceinline__ unsigned lane_off(int inst, int lane) {
+  // byte offset, from the first row of piece `inst`, of the chunk that `lane` fetches
+  __device__ static __forceinline__ unsigned lane_off(int inst, int lane, int stride) {
     const int L = inst * 64 + lane;
     const int row = L / CPR, cpos = L % CPR;
-    return (unsigned)((row * COLS + ((cpos ^ swz_f<CPR>(row)) << 3) - inst * 512) * 2);
+    return (unsigned)(((row - inst * RPP) * stride + ((cpos ^ swz_f<CPR>(row)) << 3)) * 2);
   }
   // number of instructions wave `wave` issues for one tile
   __device__ static __forceinline__ int count(int wave) {
@@ -192,19 +193,21 @@ struct AsyncTile {
     for (int k = 0; k < PER; ++k) n += (wave + NW * k < NINST) ? 1 : 0;
     return n;
   }
-  // issues this wave's instructions k0 .. k1-1 (of PER) for the tile; `off0` = lane_off(wave, lane)
+  // issues this wave's instructions k0 .. k1-1 (of PER) for the tile; `off0` = lane_off(wave, lane, stride)
   template <int K0 = 0, int K1 = PER>
-  __device__ static __forceinline__ void issue_at(const half_t* gtile, half_t* lds_tile, int wave, int lane, unsigned off0) {
+  __device__ static __forceinline__ void issue_at(const half_t* gtile, half_t* lds_tile, int wave, int lane, unsigned off0,
+                                                  int stride) {
 #pragma unroll
     for (int k = K0; k < K1; ++k) {
       const int inst = wave + NW * k;
       if (NINST % NW == 0 || inst < NINST)
-        async_copy16(gtile + inst * 512, kOneOffset ? off0 : lane_off(inst, lane), lds_tile + inst * 512);
+        async_copy16(gtile + (size_t)(inst * RPP) * stride, kOneOffset ? off0 : lane_off(inst, lane, stride),
+                     lds_tile + inst * 512);
     }
   }
   template <int K0 = 0, int K1 = PER>
-  __device__ static __forceinline__ void issue(const half_t* gtile, half_t* lds_tile, int wave, int lane) {
-    issue_at<K0, K1>(gtile, lds_tile, wave, lane, lane_off(wave, lane));
+  __device__ static __forceinline__ void issue(const half_t* gtile, half_t* lds_tile, int wave, int lane, int stride = COLS) {
+    issue_at<K0, K1>(gtile, lds_tile, wave, lane, lane_off(wave, lane, stride), stride);
   }
 };
 

@@ -69,8 +69,10 @@ void fwd_kernel(FwdParams p) {
     const int tile = xcd_remap(blockIdx.x, gridDim.x);
     bh = tile / n_qt; qt = tile % n_qt;
   }
-  const size_t qk_base = (size_t)bh * p.N * D;
-  const size_t v_base = (size_t)bh * p.N * DV;
+  // element offsets of the unit's first row and the row strides of its tensors
+  const size_t qk_base = da_abi::unit_base(p, p.sqk, bh);
+  const size_t v_base = da_abi::unit_base(p, p.sv, bh);
+  const int qk_n = (int)p.sqk.n, v_n = (int)p.sv.n;
   const int qrow0 = qt * BM + qw * 32 * QS + j;   // this lane's query row of block qs is qrow0 + 32*qs
 
   // Q fragments (B operand): column j = this lane's query, k = 8g..8g+7 of each 16-wide k-step.
@@ -80,7 +82,7 @@ void fwd_kernel(FwdParams p) {
     const float c = p.sm_scale * kLog2e;
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
-      const half_t* r = (st ? p.q2 : p.q1) + qk_base + (size_t)(qrow0 + 32 * qs) * D + 8 * g;
+      const half_t* r = (st ? p.q2 : p.q1) + qk_base + (size_t)(qrow0 + 32 * qs) * qk_n + 8 * g;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         h8 q = *reinterpret_cast<const h8*>(r + 16 * ks);
@@ -119,10 +121,11 @@ void fwd_kernel(FwdParams p) {
   const int n_tiles = CAUSAL ? (qt + 1) * (BM / BN) : p.N / BN;
   static_assert(BM % (2 * BN) == 0, "an even number of key tiles per query block");
   constexpr int VH = (VTile::PER + 1) / 2;   // V instructions are issued in two groups
-  auto load_k1 = [&](int tk, int buf) { KTile::issue(gk1 + (size_t)tk * BN * D, sKbuf + buf * C::K_BUF, wave, lane); };
-  auto load_k2 = [&](int tk, int buf) { KTile::issue(gk2 + (size_t)tk * BN * D, sKbuf + buf * C::K_BUF + C::K_TILE, wave, lane); };
-  auto load_va = [&](int tv, int buf) { VTile::template issue<0, VH>(gv + (size_t)tv * BN * DV, sVbuf + buf * C::V_TILE, wave, lane); };
-  auto load_vb = [&](int tv, int buf) { VTile::template issue<VH, VTile::PER>(gv + (size_t)tv * BN * DV, sVbuf + buf * C::V_TILE, wave, lane); };
+  const unsigned k_off = KTile::lane_off(wave, lane, qk_n), v_off = VTile::lane_off(wave, lane, v_n);
+  auto load_k1 = [&](int tk, int buf) { KTile::issue_at(gk1 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF, wave, lane, k_off, qk_n); };
+  auto load_k2 = [&](int tk, int buf) { KTile::issue_at(gk2 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF + C::K_TILE, wave, lane, k_off, qk_n); };
+  auto load_va = [&](int tv, int buf) { VTile::template issue_at<0, VH>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n); };
+  auto load_vb = [&](int tv, int buf) { VTile::template issue_at<VH, VTile::PER>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n); };
 
   // A-fragments of K for all k-steps of all 32-key tiles: row kt*32 + j, halfs 16ks + 8g .. +7
   auto read_k = [&](const half_t* sK, h8 (&ka)[NKT][NKS]) {
@@ -334,14 +337,14 @@ void fwd_kernel(FwdParams p) {
       }
     (void)qs;
   };
-  auto store_rows = [&](half_t* gbase /* first of this wave's 32 rows */) {
+  auto store_rows = [&](half_t* gbase /* first of this wave's 32 rows */, size_t row_stride) {
     constexpr int LPR = DV / 8;            // lanes per row
     constexpr int RPI = 64 / LPR;          // rows per instruction
 #pragma unroll
     for (int k = 0; k < 32 / RPI; ++k) {
       const int row = k * RPI + lane / LPR, ch = lane % LPR;
       const u32x4 v = *reinterpret_cast<const u32x4*>(stg_own + row * SROW + 8 * ch);
-      *reinterpret_cast<u32x4*>(gbase + (size_t)row * DV + 8 * ch) = v;
+      *reinterpret_cast<u32x4*>(gbase + (size_t)row * row_stride + 8 * ch) = v;
     }
   };
 
@@ -357,7 +360,7 @@ void fwd_kernel(FwdParams p) {
   if (st == 1) stage_rows(0, o[0], inv);
   __syncthreads();
   if (st == 1) {
-    if (p.u2) store_rows(p.u2 + wave_row0 * DV);
+    if (p.u2) store_rows(p.u2 + wave_row0 * DV, DV);
   } else {
     const float lam = da_abi::lambda_of_unit(p, bh);
     const half_t* stg_u2 = smem + (size_t)(wave + NW / 2) * 32 * SROW;
@@ -383,7 +386,7 @@ void fwd_kernel(FwdParams p) {
     }
     stage_rows(0, o[0], scale);
     __builtin_amdgcn_wave_barrier();   // the rows are read back by other lanes of this wave only
-    store_rows(p.y + wave_row0 * DV);
+    store_rows(p.y + da_abi::unit_base(p, p.sy, bh) + (size_t)(qt * BM + qw * 32) * (size_t)p.sy.n, (size_t)p.sy.n);
   }
 }
 

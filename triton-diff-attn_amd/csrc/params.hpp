@@ -6,6 +6,9 @@
 // One definition serves both builds of the kernels: T is the 16-bit element type of the tensors.
 namespace da_abi {
 
+// Element strides of a [B,H,N,C] tensor whose last dimension is contiguous.
+struct Strides { long long b, h, n; };
+
 template <class T>
 struct FwdParamsT {
   const T* q1; const T* q2; const T* k1; const T* k2; const T* v;
@@ -21,6 +24,7 @@ struct FwdParamsT {
   int n_keys;                   // keys n_keys..N-1 are padding and are ignored (N when there is none)
   int H;                        // heads per batch entry: unit bh belongs to head bh % H
   int lambda_stride;            // 0: lambda_scale[0] for every head; 1: lambda_scale[head]
+  Strides sqk, sv, sy;          // layouts of q1,q2,k1,k2 / v / y; u2 and the row statistics are dense
 };
 
 template <class T>
@@ -45,12 +49,19 @@ struct BwdParamsT {
   unsigned stages;              // bit 0 row preprocess, 1 d(lambda) reduce, 2 dK/dV, 3 dQ
   int H;                        // heads per batch entry: unit bh belongs to head bh % H
   int lambda_stride;            // 0: one lambda; 1: one per head
+  Strides sqk, sv, sy, sdy;     // layouts of q1,q2,k1,k2 / v / y / dy; everything else is dense
 };
 
 // lambda of the (batch, head) unit bh
 template <class P>
 __device__ __forceinline__ float lambda_of_unit(const P& p, int bh) {
   return (float)p.lambda_scale[(bh % p.H) * p.lambda_stride];
+}
+
+// offset in elements of the first row of the (batch, head) unit bh
+template <class P>
+__device__ __forceinline__ size_t unit_base(const P& p, const Strides& s, int bh) {
+  return (size_t)(bh / p.H) * (size_t)s.b + (size_t)(bh % p.H) * (size_t)s.h;
 }
 
 }  // namespace da_abi

@@ -51,10 +51,31 @@ def _check_inputs(Q1, Q2, K1, K2, V):
 
 
 def _pad_rows(t, n_pad):
-    """[B,H,N,C] -> dense [B,H,n_pad,C] with zero rows appended (the tensor itself when nothing is missing)."""
-    if t.size(2) == n_pad:
-        return t.contiguous()
+    """[B,H,N,C] -> dense [B,H,n_pad,C] with zero rows appended."""
     return torch.nn.functional.pad(t, (0, 0, 0, n_pad - t.size(2)))
+
+
+def _strides_ok(t):
+    """Whether the kernels can read t in place: contiguous rows, every other stride a non-negative
+    multiple of 8 elements (16-byte aligned rows), base pointer 16-byte aligned."""
+    sb, sh, sn, sc = t.stride()
+    return (sc == 1 and sn >= t.size(3) and sn % 8 == 0 and sb % 8 == 0 and sh % 8 == 0 and sb >= 0 and sh >= 0
+            and sn <= (1 << 26) and t.data_ptr() % 16 == 0)
+
+
+def _in_place(t):
+    """t itself when the kernels can read it through its strides, else a dense copy."""
+    return t if _strides_ok(t) else t.contiguous()
+
+
+def _is_dense(t):
+    B, H, N, C = t.shape
+    return t.stride() == (H * N * C, N * C, C, 1)
+
+
+def _current_stream(dev):
+    """Raw handle of torch's current stream on dev (no Stream object is built)."""
+    return torch._C._cuda_getCurrentRawStream(dev.index if dev.index is not None else torch._C._cuda_getDevice())
 
 
 def _lambda_tensor(lambda_scale, device, dtype=torch.float16, num_heads=1):
@@ -83,28 +104,48 @@ class _diff_attention(torch.autograd.Function):
         # lengths are padded with zero rows here; forward and backward ignore the padding keys, and a
         # padded query row has a zero upstream gradient, so it adds nothing to dK and dV.
         n_pad = -(-N // _SEQ_MULTIPLE) * _SEQ_MULTIPLE
-        q1, q2, k1, k2, v = (_pad_rows(t, n_pad) for t in (Q1, Q2, K1, K2, V))
+        if n_pad != N:
+            q1, q2, k1, k2, v = (_pad_rows(t, n_pad) for t in (Q1, Q2, K1, K2, V))
+        else:
+            # Tensors are read through their strides (the reference passes Q1's and V's to its kernel,
+            # src/kernel.py:487-494): a [B,N,H,d] projection output viewed as [B,H,N,d] is not copied.
+            # The four q/k tensors share one set of strides, as in the reference.
+            q1, q2, k1, k2, v = (_in_place(t) for t in (Q1, Q2, K1, K2, V))
+            if not (q1.stride() == q2.stride() == k1.stride() == k2.stride()):
+                q1, q2, k1, k2 = (t.contiguous() for t in (q1, q2, k1, k2))
         lam = _lambda_tensor(LAMBDA_SCALE, dev, Q1.dtype, H)
         rms_norm = bool(rms_norm)
         flags = ((_FLAG_RMS_NORM if rms_norm else 0) | (_FLAG_CAUSAL if causal else 0)
                  | (_FLAG_BF16 if Q1.dtype == torch.bfloat16 else 0)
                  | (_FLAG_LAMBDA_PER_HEAD if lam.numel() > 1 else 0))
 
-        y = torch.empty_like(v)
+        y = torch.empty_like(v)         # v's layout when v is a permuted dense buffer, else dense
+        layout = None
+        if not (_is_dense(q1) and _is_dense(v) and _is_dense(y)):
+            layout = _native.Layout(*q1.stride()[:3], *v.stride()[:3], *y.stride()[:3], *y.stride()[:3])
         # what only a backward reads (src/kernel.py:505 saves its counterparts unconditionally) is neither
         # allocated nor written when no input asks for a gradient, e.g. under torch.no_grad()
         differentiable = any(ctx.needs_input_grad)
-        u2 = torch.empty_like(v) if differentiable else None
-        stat = lambda: torch.empty((B, H, n_pad), device=dev, dtype=torch.float32)
-        lse1, lse2 = (stat(), stat()) if differentiable else (None, None)
-        rinv = stat() if (rms_norm and differentiable) else None
+        u2 = lse1 = lse2 = rinv = None
+        if differentiable:
+            u2 = torch.empty((B, H, n_pad, 2 * D), device=dev, dtype=v.dtype)
+            # the two logsumexps and the RMSNorm statistic share one allocation
+            stats = torch.empty((3 if rms_norm else 2, B, H, n_pad), device=dev, dtype=torch.float32)
+            lse1, lse2 = stats[0], stats[1]
+            rinv = stats[2] if rms_norm else None
 
-        with torch.cuda.device(dev):
-            stream = torch.cuda.current_stream().cuda_stream
-            _native.check(lib.diffattn_forward_padded(
+        if dev.index is not None and dev.index != torch._C._cuda_getDevice():
+            with torch.cuda.device(dev):
+                rc = lib.diffattn_forward_padded(
+                    q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
+                    lam.data_ptr(), y.data_ptr(), _ptr(u2), _ptr(lse1), _ptr(lse2), _ptr(rinv),
+                    B, H, n_pad, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, layout, _current_stream(dev))
+        else:
+            rc = lib.diffattn_forward_padded(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
                 lam.data_ptr(), y.data_ptr(), _ptr(u2), _ptr(lse1), _ptr(lse2), _ptr(rinv),
-                B, H, n_pad, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, stream))
+                B, H, n_pad, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, layout, _current_stream(dev))
+        _native.check(rc)
 
         if differentiable:
             ctx.save_for_backward(q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam)
@@ -119,13 +160,16 @@ class _diff_attention(torch.autograd.Function):
     @once_differentiable        # the gradients are plain kernel outputs: a second derivative raises
     def backward(ctx, dO):
         q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam = ctx.saved_tensors
-        B, H, N, D = q1.shape
+        B, H, N, D = q1.shape           # N is the padded length here
         lib = _native.lib()
         dev = q1.device
+        n_valid = ctx.N_VALID
         if dO.dtype != q1.dtype:
             dO = dO.to(q1.dtype)
-        dO = _pad_rows(dO, N)           # N is the padded length here
-        n_valid = ctx.N_VALID
+        dO = _pad_rows(dO, N) if n_valid != N else _in_place(dO)
+        layout = None
+        if not (_is_dense(q1) and _is_dense(v) and _is_dense(y) and _is_dense(dO)):
+            layout = _native.Layout(*q1.stride()[:3], *v.stride()[:3], *y.stride()[:3], *dO.stride()[:3])
 
         # only the kernels whose outputs some input asked for are launched (stage bits of the C ABI:
         # 1 row preprocess, 2 d(lambda) reduction, 4 dK/dV, 8 dQ)
@@ -133,19 +177,35 @@ class _diff_attention(torch.autograd.Function):
         want_q, want_kv = need[0] or need[1], need[2] or need[3] or need[4]
         want_lam = ctx.lambda_meta is not None and need[6]
         stages = 1 | (2 if want_lam else 0) | (4 if want_kv else 0) | (8 if want_q else 0)
-        dq1, dq2 = (torch.empty_like(q1), torch.empty_like(q2)) if want_q else (None, None)
-        dk1, dk2, dv = (torch.empty_like(k1), torch.empty_like(k2), torch.empty_like(v)) if want_kv else (None,) * 3
+        # gradients are dense [B,H,N,.] whatever the layout of the inputs; those of equal shape share
+        # one allocation
+        dq1 = dq2 = dk1 = dk2 = dv = None
+        n_qk = (2 if want_q else 0) + (2 if want_kv else 0)
+        if n_qk:
+            gqk = torch.empty((n_qk, B, H, N, D), device=dev, dtype=q1.dtype)
+            if want_q:
+                dq1, dq2 = gqk[0], gqk[1]
+            if want_kv:
+                dk1, dk2 = gqk[n_qk - 2], gqk[n_qk - 1]
+                dv = torch.empty((B, H, N, 2 * D), device=dev, dtype=q1.dtype)
         dlam = torch.empty(lam.numel(), device=dev, dtype=q1.dtype) if want_lam else None
         ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D, ctx.FLAGS)
         ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
 
-        with torch.cuda.device(dev):
-            stream = torch.cuda.current_stream().cuda_stream
-            _native.check(lib.diffattn_backward_stages(
+        def launch():
+            return lib.diffattn_backward_stages(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv), dO.data_ptr(),
                 _ptr(dq1), _ptr(dq2), _ptr(dk1), _ptr(dk2), _ptr(dv), _ptr(dlam),
-                ws.data_ptr(), ws_bytes, B, H, N, n_valid, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stages, stream))
+                ws.data_ptr(), ws_bytes, B, H, N, n_valid, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stages,
+                layout, _current_stream(dev))
+
+        if dev.index is not None and dev.index != torch._C._cuda_getDevice():
+            with torch.cuda.device(dev):
+                rc = launch()
+        else:
+            rc = launch()
+        _native.check(rc)
 
         dlambda = None
         if want_lam:

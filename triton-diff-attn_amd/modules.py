@@ -64,8 +64,9 @@ class DiffAttn(nn.Module):
         k = self.k_proj(x).view(B, N, H, 2, d).permute(3, 0, 2, 1, 4)
         v = self.v_proj(x).view(B, N, H, 2 * d).transpose(1, 2)
         lam = self.lambda_scale().to(x.dtype)
-        heads = self.attention(q[0].contiguous(), q[1].contiguous(), k[0].contiguous(), k[1].contiguous(),
-                               v.contiguous(), lambda_scale=lam, lambda_init=self.lambda_init, rms_norm=True,
+        # views of the projection outputs: the operator reads them through their strides and returns the
+        # heads in v's [B,N,H,2d] memory layout, so neither side of it copies
+        heads = self.attention(q[0], q[1], k[0], k[1], v, lambda_scale=lam, lambda_init=self.lambda_init, rms_norm=True,
                                **({"causal": True} if self.causal else {}))
         heads = heads * self.head_gain
         return self.out_proj(heads.transpose(1, 2).reshape(B, N, E))
