@@ -209,7 +209,7 @@ def main():
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(), dy.data_ptr(),
                 *[g.data_ptr() for g in grads], dlam.data_ptr(), ws.data_ptr(), ws_bytes,
-                B, H, N, N, D, sm, cfg["lambda_init"], flags, mask, None, stream))
+                B, H, N, N, D, sm, cfg["lambda_init"], flags, mask, None, None, stream))
 
         launch_forward()
         k_iters = max(5, min(args.steps, 30))

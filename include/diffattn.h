@@ -35,6 +35,7 @@ extern "C" {
 #define DIFFATTN_EINVAL_ALIGN (-5)  /* a pointer is not 16-byte aligned */
 #define DIFFATTN_EINVAL_FLAGS (-6)  /* unknown bits in `flags` */
 #define DIFFATTN_EINVAL_SCRATCH (-7) /* problem too large for diffattn_backward_static */
+#define DIFFATTN_EINVAL_DROPOUT (-9) /* dropout probability outside [0, 255/256] */
 #define DIFFATTN_EINVAL_LAYOUT (-8)  /* a stride in diffattn_layout is negative, not a multiple of 8, or a row stride is below the row width */
 
 /* `flags` of the forward and backward entry points.  DIFFATTN_RMS_NORM is the reference's boolean
@@ -70,6 +71,22 @@ typedef struct diffattn_layout {
   long long dy_b, dy_h, dy_n;   /* dy, backward only (C = 2D); ignored by the forward */
 } diffattn_layout;
 
+/*
+ * Dropout on the two softmax maps.  No counterpart in the reference, which lists dropout as
+ * missing (src/kernel.py:4, README.md:2).  Each (query, key) pair of each softmax stream is
+ * dropped independently with probability p before the product with v, and the kept probabilities
+ * are scaled by 1/(1-p), as torch's scaled_dot_product_attention does for its single map:
+ *     x = (drop(softmax(s q1 k1^T)) - lambda drop'(softmax(s q2 k2^T))) v.
+ * The decisions are a pure function of (seed, stream, batch*head unit, query, key, N): forward and
+ * backward of one problem must be given the same struct, and diffattn_dropout_mask writes the same
+ * decisions out.  p is used in steps of 1/256 (rounded to the nearest; the scale uses the rounded
+ * value); p = 0 or a NULL pointer means no dropout.
+ */
+typedef struct diffattn_dropout {
+  float p;                      /* drop probability, 0 <= p <= 255/256 */
+  unsigned long long seed;
+} diffattn_dropout;
+
 /* ABI version of this header; bumped when a signature changes. */
 int diffattn_abi_version(void);
 
@@ -99,12 +116,13 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
  * n_valid..N-1 of the outputs are to be discarded.  The matching backward is
  * diffattn_backward_stages with the same n_valid, on the padded tensors with zero rows of dy in the
  * padding; it returns the gradients of rows 0..n_valid-1.  diffattn_forward is this function with
- * n_valid = N.  `layout` gives the strides of q1, q2, k1, k2, v and y (NULL: all dense).
+ * n_valid = N.  `layout` gives the strides of q1, q2, k1, k2, v and y (NULL: all dense);
+ * `dropout` switches dropout on (NULL: none).
  */
 int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
                             const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
                             int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
-                            const diffattn_layout* layout, void* stream);
+                            const diffattn_layout* layout, const diffattn_dropout* dropout, void* stream);
 
 /* Bytes of device workspace diffattn_backward needs for this problem size and these flags (0 on bad
  * sizes or unknown flag bits).  Counterpart of the scratch tensors the reference's backward
@@ -144,7 +162,7 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
  * n_valid (1..N) is the real sequence length of a problem that went through
  * diffattn_forward_padded (N when there is no padding): keys n_valid..N-1 are ignored.
  * `layout` gives the strides of q1, q2, k1, k2, v, y and dy (NULL: all dense); the gradients are
- * written dense.
+ * written dense.  `dropout` must be what the forward was given.
  */
 #define DIFFATTN_STAGE_PREP 1u
 #define DIFFATTN_STAGE_DLAMBDA 2u
@@ -157,7 +175,17 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                              void* workspace, size_t workspace_bytes,
                              int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
-                             unsigned stage_mask, const diffattn_layout* layout, void* stream);
+                             unsigned stage_mask, const diffattn_layout* layout, const diffattn_dropout* dropout,
+                             void* stream);
+
+/*
+ * Writes the keep decisions of `dropout` for softmax stream 0 or 1 of a [B,H,N,N] problem as bytes
+ * (1 kept, 0 dropped) to `keep` (device memory, B*H*N*N bytes).  N is the padded length the
+ * kernels are called with.  No counterpart in the reference; it lets a test hand the very masks
+ * the kernels use to a reference implementation.
+ */
+int diffattn_dropout_mask(unsigned char* keep, int B, int H, int N, int softmax_stream, const diffattn_dropout* dropout,
+                          void* stream);
 
 /*
  * Backward without a workspace argument and without any allocation.  No counterpart in the

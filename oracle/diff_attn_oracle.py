@@ -58,12 +58,16 @@ def normalise(x, lambda_init):
     return (1 - lambda_init) * (x * rinv), rinv
 
 
-def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False, causal=False):
+def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False, causal=False,
+                 keep1=None, keep2=None, dropout_p=0.0):
     """One or more (b, h) units: tensors [..., N, D] / [..., N, 2D], already in the work dtype.
 
     Follows src/layers.py:60-78 line for line (minus the .half() casts).  `causal` (not in the
     reference, which lists masking as missing, src/kernel.py:4) lets query i see keys 0..i only, in
-    both softmax streams.
+    both softmax streams.  Dropout (likewise listed as missing) takes its decisions as arguments,
+    so the oracle stays deterministic: `keep1`, `keep2` [..., N, N] (non-zero = kept) multiply the
+    two softmax maps after normalisation, and the kept entries are scaled by 1 / (1 - dropout_p),
+    as torch's scaled_dot_product_attention defines dropout for its single map.
     """
     head_dim = q1.size(-1)
     sm_scale = 1 / math.sqrt(head_dim)                       # src/layers.py:60-62
@@ -76,6 +80,10 @@ def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False, 
         s2 = s2.masked_fill(future, float("-inf"))
     p1 = torch.softmax(s1, dim=-1)                           # src/layers.py:65
     p2 = torch.softmax(s2, dim=-1)                           # src/layers.py:68
+    if keep1 is not None:
+        p1 = p1 * keep1.to(p1.dtype) / (1 - dropout_p)
+    if keep2 is not None:
+        p2 = p2 * keep2.to(p2.dtype) / (1 - dropout_p)
     p = p1 - lam * p2                                        # src/layers.py:70
     x = torch.matmul(p, v)                                   # src/layers.py:72
     if rms_norm:                                             # src/layers.py:74-78
@@ -97,22 +105,25 @@ def forward_unit(q1, q2, k1, k2, v, lam, lambda_init, rms_norm, want_aux=False, 
 
 
 def forward(q1, q2, k1, k2, v, lambda_scale, lambda_init=0.8, rms_norm=False,
-            dtype=torch.float32, chunk=8, want_aux=False, causal=False):
+            dtype=torch.float32, chunk=8, want_aux=False, causal=False, keep1=None, keep2=None, dropout_p=0.0):
     """Differential attention forward, [B,H,N,D] inputs, result in `dtype`.
 
     Inputs are upcast (fp16 values are used exactly as rounded).  `chunk` = number of (b,h)
-    units processed together.
+    units processed together.  keep1, keep2: [B,H,N,N] dropout decisions (see forward_unit).
     """
     B, H, N, D = q1.shape
     Dv = v.shape[-1]
     f = lambda t: t.reshape(B * H, N, t.shape[-1]).to(dtype)
     q1f, q2f, k1f, k2f, vf = f(q1), f(q2), f(k1), f(k2), f(v)
+    m1 = None if keep1 is None else keep1.reshape(B * H, N, N)
+    m2 = None if keep2 is None else keep2.reshape(B * H, N, N)
     lam_values = _lambda_values(lambda_scale, H, dtype)
     ys, auxs = [], []
     for s in range(0, B * H, chunk):
         sl = slice(s, s + chunk)
         lam = _lambda_of_units(lam_values, torch.arange(s, min(s + chunk, B * H)), H)
-        r = forward_unit(q1f[sl], q2f[sl], k1f[sl], k2f[sl], vf[sl], lam, lambda_init, rms_norm, want_aux, causal)
+        r = forward_unit(q1f[sl], q2f[sl], k1f[sl], k2f[sl], vf[sl], lam, lambda_init, rms_norm, want_aux, causal,
+                         None if m1 is None else m1[sl], None if m2 is None else m2[sl], dropout_p)
         if want_aux:
             ys.append(r[0]); auxs.append(r[1])
         else:
@@ -131,7 +142,7 @@ def forward(q1, q2, k1, k2, v, lambda_scale, lambda_init=0.8, rms_norm=False,
 
 
 def forward_backward(q1, q2, k1, k2, v, lambda_scale, dy, lambda_init=0.8, rms_norm=False,
-                     dtype=torch.float32, chunk=8, causal=False):
+                     dtype=torch.float32, chunk=8, causal=False, keep1=None, keep2=None, dropout_p=0.0):
     """Forward + autograd backward of the restated graph.
 
     Returns (y, dq1, dq2, dk1, dk2, dv, dlambda) in `dtype`; dlambda has shape [1] and is the sum
@@ -144,6 +155,8 @@ def forward_backward(q1, q2, k1, k2, v, lambda_scale, dy, lambda_init=0.8, rms_n
     ins = [f(q1), f(q2), f(k1), f(k2), f(v)]
     dyf = f(dy)
     lam0 = _lambda_values(lambda_scale, H, dtype)
+    m1 = None if keep1 is None else keep1.reshape(B * H, N, N)
+    m2 = None if keep2 is None else keep2.reshape(B * H, N, N)
     grads = [torch.empty_like(t) for t in ins]
     dlam = torch.zeros_like(lam0)
     ys = []
@@ -152,7 +165,8 @@ def forward_backward(q1, q2, k1, k2, v, lambda_scale, dy, lambda_init=0.8, rms_n
         leaves = [t[sl].detach().clone().requires_grad_(True) for t in ins]
         lam_leaf = lam0.detach().clone().requires_grad_(True)
         lam = _lambda_of_units(lam_leaf, torch.arange(s, min(s + chunk, B * H)), H)
-        y = forward_unit(*leaves, lam, lambda_init, rms_norm, causal=causal)
+        y = forward_unit(*leaves, lam, lambda_init, rms_norm, causal=causal,
+                         keep1=None if m1 is None else m1[sl], keep2=None if m2 is None else m2[sl], dropout_p=dropout_p)
         g = torch.autograd.grad(y, leaves + [lam_leaf], dyf[sl])
         for dst, src in zip(grads, g[:5]):
             dst[sl] = src

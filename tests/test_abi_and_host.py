@@ -21,7 +21,7 @@ def test_header_declares_the_expected_entry_points():
     assert declared_symbols() == sorted([
         "diffattn_abi_version", "diffattn_strerror", "diffattn_forward", "diffattn_forward_padded",
         "diffattn_backward_workspace_bytes", "diffattn_backward", "diffattn_backward_stages",
-        "diffattn_backward_static"])
+        "diffattn_backward_static", "diffattn_dropout_mask"])
 
 
 def test_library_exports_every_declared_symbol():
@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_symbols():
         assert hasattr(lib, name), name
         assert name in _native.SYMBOLS, "binding table misses %s" % name
-    assert lib.diffattn_abi_version() == 5 == _native.ABI_VERSION
+    assert lib.diffattn_abi_version() == 6 == _native.ABI_VERSION
 
 
 def test_argument_rejection_needs_no_gpu():
@@ -51,7 +51,7 @@ def test_argument_rejection_needs_no_gpu():
     bad = args(1, 1, 128, 64)
     bad[-2] = 1 << 12                             # unknown flag bit
     assert lib.diffattn_forward(*bad) == -6
-    padded = lambda n_valid, layout=None: [p] * 11 + [1, 1, 128, n_valid, 64, 0.125, 0.8, 1, layout, None]
+    padded = lambda n_valid, layout=None, drop=None: [p] * 11 + [1, 1, 128, n_valid, 64, 0.125, 0.8, 1, layout, drop, None]
     assert lib.diffattn_forward_padded(*padded(0)) == -3
     assert lib.diffattn_forward_padded(*padded(129)) == -3
     assert lib.diffattn_backward_workspace_bytes(1, 1, 100, 64, 0) == 0
@@ -64,7 +64,7 @@ def test_argument_rejection_needs_no_gpu():
     assert lib.diffattn_backward(*bargs) == -4
     bargs[19], bargs[-2] = need, 1 << 12
     assert lib.diffattn_backward(*bargs) == -6
-    sargs = lambda n_valid, layout=None: bargs[:23] + [n_valid, 64, 0.125, 0.8, 1, 15, layout, None]
+    sargs = lambda n_valid, layout=None, drop=None: bargs[:23] + [n_valid, 64, 0.125, 0.8, 1, 15, layout, drop, None]
     assert lib.diffattn_backward_stages(*sargs(0)) == -3
     assert lib.diffattn_backward_stages(*sargs(257)) == -3
     # strides: multiples of 8 elements, rows at least as far apart as they are wide
@@ -74,7 +74,13 @@ def test_argument_rejection_needs_no_gpu():
         lay = _native.Layout(**dict(good, **{field: value}))
         assert lib.diffattn_forward_padded(*padded(128, ctypes.byref(lay))) == -8, field
         assert lib.diffattn_backward_stages(*sargs(256, ctypes.byref(lay))) == -8, field
-    for code in (0, -1, -2, -3, -4, -5, -6, -7, -8):
+    for bad_p in (-0.1, 1.0, float("nan")):
+        drop = _native.Dropout(bad_p, 1)
+        assert lib.diffattn_forward_padded(*padded(128, None, ctypes.byref(drop))) == -9, bad_p
+        assert lib.diffattn_backward_stages(*sargs(256, None, ctypes.byref(drop))) == -9, bad_p
+    assert lib.diffattn_dropout_mask(p, 1, 1, 128, 2, ctypes.byref(_native.Dropout(0.5, 1)), None) == -2     # stream 0 or 1
+    assert lib.diffattn_dropout_mask(p, 1, 1, 128, 0, None, None) == -1
+    for code in (0, -1, -2, -3, -4, -5, -6, -7, -8, -9):
         assert len(lib.diffattn_strerror(code)) > 0
 
 
@@ -119,14 +125,15 @@ def test_drop_in_signature_matches_reference():
     import layers
     from kernel import _diff_attention
     sig = inspect.signature(layers.MultiheadDiffAttnKernel)
-    # the reference's eight parameters in the reference's order; `causal` is an addition at the end
-    assert list(sig.parameters) == ["q1", "q2", "k1", "k2", "v", "lambda_scale", "lambda_init", "rms_norm", "causal"]
-    assert sig.parameters["causal"].default is False
+    # the reference's eight parameters in the reference's order; the additions follow at the end
+    assert list(sig.parameters) == ["q1", "q2", "k1", "k2", "v", "lambda_scale", "lambda_init", "rms_norm", "causal",
+                                    "dropout_p", "dropout_seed"]
+    assert sig.parameters["causal"].default is False and sig.parameters["dropout_p"].default == 0.0
     assert sig.parameters["lambda_scale"].default == -0.5
     assert sig.parameters["lambda_init"].default == 0.8
     assert sig.parameters["rms_norm"].default is False
     fsig = inspect.signature(_diff_attention.forward)
     assert list(fsig.parameters) == ["ctx", "Q1", "Q2", "K1", "K2", "V", "SM_SCALE", "LAMBDA_SCALE", "LAMBDA_INIT", "rms_norm",
-                                     "causal"]
+                                     "causal", "dropout_p", "dropout_seed"]
     assert fsig.parameters["causal"].default is False
     assert issubclass(_diff_attention, torch.autograd.Function)

@@ -129,3 +129,20 @@ def test_per_head_lambda_layer_with_the_kernel_matches_the_stock_operator():
     for (name, pf), (_, ps) in zip(fused.named_parameters(), stock.named_parameters()):
         scale = ps.grad.float().abs().max().item()
         assert (pf.grad.float() - ps.grad.float()).abs().max().item() <= 5e-2 * scale + 1e-3, name
+
+
+@pytest.mark.gpu
+def test_attention_dropout_acts_in_training_mode_only():
+    torch.manual_seed(6)
+    dev = torch.device("cuda:0")
+    layer = modules.DiffAttn(256, 2, attention_dropout=0.3, device=dev)
+    x = (0.5 * torch.randn(2, 128, 256, device=dev)).half()
+    layer.eval()
+    a, b = layer(x), layer(x)
+    assert torch.equal(a, b)
+    layer.train()
+    c, d = layer(x), layer(x)
+    assert not torch.equal(c, d) and not torch.equal(c, a)      # fresh masks per call
+    assert torch.isfinite(c).all()
+    c.float().square().mean().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in layer.parameters())

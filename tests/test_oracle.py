@@ -205,3 +205,76 @@ def test_per_head_lambda_is_the_scalar_oracle_head_by_head():
                 for a, b in zip(full[:6], one[:6]):
                     assert torch.allclose(a[sl], b, rtol=0, atol=1e-12)
                 assert torch.allclose(full[6][h], one[6][0], rtol=1e-12, atol=1e-12)
+
+
+# ---- dropout (explicit keep decisions) ---------------------------------------------------------------
+
+def _keep_masks(B, H, N, p, seed):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.rand(B, H, N, N, generator=g) >= p), (torch.rand(B, H, N, N, generator=g) >= p)
+
+
+def test_dropout_keeping_everything_only_rescales():
+    q1, q2, k1, k2, v = rand_inputs(1, 2, 12, 4, seed=30)
+    ones = torch.ones(1, 2, 12, 12, dtype=torch.bool)
+    plain = orc.forward(q1, q2, k1, k2, v, 0.4, rms_norm=False, dtype=torch.float64)
+    kept = orc.forward(q1, q2, k1, k2, v, 0.4, rms_norm=False, dtype=torch.float64, keep1=ones, keep2=ones, dropout_p=0.25)
+    assert torch.allclose(kept, plain / 0.75, atol=1e-12)
+    # with the norm the scale cancels (up to eps)
+    a = orc.forward(q1, q2, k1, k2, v, 0.4, rms_norm=True, dtype=torch.float64)
+    b = orc.forward(q1, q2, k1, k2, v, 0.4, rms_norm=True, dtype=torch.float64, keep1=ones, keep2=ones, dropout_p=0.25)
+    assert torch.allclose(a, b, atol=1e-4)
+
+
+def test_dropping_a_key_everywhere_is_zeroing_its_value_row():
+    """Dropout acts after the softmax normalisation: dropping key j for every query, in both maps, removes
+    v[j] from every output row without renormalising the other weights."""
+    q1, q2, k1, k2, v = rand_inputs(2, 2, 10, 4, seed=31)
+    keep = torch.ones(2, 2, 10, 10, dtype=torch.bool)
+    keep[:, :, :, 3] = False
+    keep[:, :, :, 7] = False
+    got = orc.forward(q1, q2, k1, k2, v, 0.6, rms_norm=False, dtype=torch.float64, keep1=keep, keep2=keep, dropout_p=0.2)
+    v0 = v.clone()
+    v0[:, :, 3] = 0
+    v0[:, :, 7] = 0
+    want = orc.forward(q1, q2, k1, k2, v0, 0.6, rms_norm=False, dtype=torch.float64) / 0.8
+    assert torch.allclose(got, want, atol=1e-12)
+
+
+def test_dropout_masks_act_on_their_own_stream():
+    """With lambda = 0 the second map's mask is irrelevant; with only the second map dropped entirely the
+    result is the first map's attention alone."""
+    q1, q2, k1, k2, v = rand_inputs(1, 2, 9, 4, seed=32)
+    m1, m2 = _keep_masks(1, 2, 9, 0.3, seed=33)
+    a = orc.forward(q1, q2, k1, k2, v, 0.0, dtype=torch.float64, keep1=m1, keep2=m2, dropout_p=0.3)
+    b = orc.forward(q1, q2, k1, k2, v, 0.0, dtype=torch.float64, keep1=m1, keep2=~m2, dropout_p=0.3)
+    assert torch.equal(a, b)
+    none = torch.zeros_like(m2)
+    c = orc.forward(q1, q2, k1, k2, v, 0.9, dtype=torch.float64, keep1=torch.ones_like(m1), keep2=none, dropout_p=0.0)
+    assert torch.allclose(c, F.scaled_dot_product_attention(q1, k1, v), atol=1e-12)
+
+
+@pytest.mark.parametrize("rms", [False, True])
+def test_dropout_brute_force_f64(rms):
+    q1, q2, k1, k2, v = rand_inputs(1, 1, 7, 3, seed=34)
+    m1, m2 = _keep_masks(1, 1, 7, 0.4, seed=35)
+    y = orc.forward(q1, q2, k1, k2, v, 0.37, lambda_init=0.6, rms_norm=rms, dtype=torch.float64, keep1=m1, keep2=m2, dropout_p=0.4)
+    ref = brute_force.forward_unit(*(t[0, 0].numpy() for t in (q1, q2, k1, k2, v)), 0.37, 0.6, rms,
+                                   keep=(m1[0, 0].numpy(), m2[0, 0].numpy()), dropout_p=0.4)
+    assert np.allclose(y[0, 0].numpy(), ref, atol=1e-12)
+
+
+def test_dropout_gradients_respect_the_masks():
+    """A dropped (query, key) pair carries no gradient into v through that map: with lambda = 0, dv[j] only
+    collects the queries that kept j; and gradcheck holds with the masks in place."""
+    q1, q2, k1, k2, v = rand_inputs(1, 1, 6, 2, seed=36)
+    m1, m2 = _keep_masks(1, 1, 6, 0.5, seed=37)
+    m1[0, 0, :, 2] = False                     # nobody keeps key 2 in the first map
+    dy = torch.randn(1, 1, 6, 4, dtype=torch.float64, generator=torch.Generator().manual_seed(38))
+    out = orc.forward_backward(q1, q2, k1, k2, v, torch.tensor([0.0], dtype=torch.float64), dy, 0.8, False,
+                               dtype=torch.float64, keep1=m1, keep2=m2, dropout_p=0.5)
+    assert out[5][0, 0, 2].abs().max() == 0    # dv of key 2
+    lam = torch.tensor(0.45, dtype=torch.float64, requires_grad=True)
+    ins = [t[0].clone().requires_grad_(True) for t in (q1, q2, k1, k2, v)] + [lam]
+    fn = lambda a, b, c, d, e, l: orc.forward_unit(a, b, c, d, e, l, 0.8, True, keep1=m1[0], keep2=m2[0], dropout_p=0.5)
+    assert torch.autograd.gradcheck(fn, ins, eps=1e-6, atol=1e-6)

@@ -11,7 +11,7 @@ import torch  # noqa: F401  (must precede loading the library)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdiffattn.so")
 
-ABI_VERSION = 5   # the version of include/diffattn.h this binding is written against
+ABI_VERSION = 6   # the version of include/diffattn.h this binding is written against
 
 _lib = None
 
@@ -25,7 +25,13 @@ class Layout(ctypes.Structure):
         "qk_b", "qk_h", "qk_n", "v_b", "v_h", "v_n", "y_b", "y_h", "y_n", "dy_b", "dy_h", "dy_n")]
 
 
+class Dropout(ctypes.Structure):
+    """diffattn_dropout: drop probability and seed."""
+    _fields_ = [("p", ctypes.c_float), ("seed", ctypes.c_ulonglong)]
+
+
 _lp = ctypes.POINTER(Layout)
+_dp = ctypes.POINTER(Dropout)
 
 SYMBOLS = {
     "diffattn_abi_version": (ctypes.c_int, []),
@@ -33,14 +39,15 @@ SYMBOLS = {
     "diffattn_forward": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp] + [ctypes.c_int] * 4
                          + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
     "diffattn_forward_padded": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp] + [ctypes.c_int] * 5
-                                + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _lp, _vp]),
+                                + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _lp, _dp, _vp]),
     "diffattn_backward_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int] * 5),
     "diffattn_backward": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp, _vp] + [_vp] * 6
                           + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 4
                           + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
     "diffattn_backward_stages": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp, _vp] + [_vp] * 6
                                  + [_vp, ctypes.c_size_t] + [ctypes.c_int] * 5
-                                 + [ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_uint, _lp, _vp]),
+                                 + [ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_uint, _lp, _dp, _vp]),
+    "diffattn_dropout_mask": (ctypes.c_int, [_vp] + [ctypes.c_int] * 4 + [_dp, _vp]),
     "diffattn_backward_static": (ctypes.c_int, [_vp] * 5 + [_vp, _vp, _vp, _fp, _fp, _fp, _vp] + [_vp] * 6
                                  + [ctypes.c_int] * 4 + [ctypes.c_float, ctypes.c_float, ctypes.c_int, _vp]),
 }

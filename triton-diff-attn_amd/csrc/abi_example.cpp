@@ -79,10 +79,10 @@ int main(int argc, char** argv) {
     const diffattn_layout lay = {(long long)N * H * d, d, H * d, (long long)N * H * dv, dv, H * dv,
                                  (long long)N * H * dv, dv, H * dv, (long long)N * H * dv, dv, H * dv};
     DA_OK(diffattn_forward_padded(in[0], in[1], in[2], in[3], in[4], in[6], y, u2, lse1, lse2, rinv,
-                                  B, H, N, N, D, sm_scale, lambda_init, flags, &lay, stream));
+                                  B, H, N, N, D, sm_scale, lambda_init, flags, &lay, nullptr, stream));
     DA_OK(diffattn_backward_stages(in[0], in[1], in[2], in[3], in[4], in[6], y, u2, lse1, lse2, rinv, in[5],
                                    grad[0], grad[1], grad[2], grad[3], grad[4], grad[5], ws, ws_bytes,
-                                   B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, &lay, stream));
+                                   B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, &lay, nullptr, stream));
   } else {
     DA_OK(diffattn_forward(in[0], in[1], in[2], in[3], in[4], in[6], y, u2, lse1, lse2, rinv,
                            B, H, N, D, sm_scale, lambda_init, flags, stream));

@@ -2,6 +2,7 @@
 // workspace carve-up and kernel launches.  Nothing here allocates or synchronises; the only state
 // is the per-device address of the built-in scratch array of diffattn_backward_static.
 #include <atomic>
+#include <cstring>
 
 #include "../../include/diffattn.h"
 #include "params.hpp"
@@ -82,6 +83,34 @@ int resolve_layout(const diffattn_layout* l, int H, int N, int D, Layouts* out) 
   return DIFFATTN_OK;
 }
 
+// Dropout parameters as the kernels want them; none (threshold 0) without a request or with p = 0.
+int resolve_dropout(const diffattn_dropout* d, da_abi::DropoutCfg* out) {
+  *out = {0u, 0u, 0u, 1.0f};
+  if (!d) return DIFFATTN_OK;
+  // the range test is done on the bit pattern: this file is built with -fno-honor-nans, under which a
+  // floating-point comparison does not reject a NaN
+  unsigned bits;
+  memcpy(&bits, &d->p, sizeof bits);
+  if (bits > 0x3f7f0000u) return DIFFATTN_EINVAL_DROPOUT;      // negative, NaN, or above 255/256 = 0x3f7f0000
+  const unsigned thr = (unsigned)(d->p * 256.0f + 0.5f);
+  if (thr > 255u) return DIFFATTN_EINVAL_DROPOUT;
+  out->seed_lo = (unsigned)(d->seed & 0xffffffffull);
+  out->seed_hi = (unsigned)(d->seed >> 32);
+  out->threshold = thr;
+  out->keep_scale = 256.0f / (float)(256u - thr);
+  return DIFFATTN_OK;
+}
+
+// keep[bh][q][k] = 1 if the pair survives dropout in softmax stream `stream`, else 0
+__global__ __launch_bounds__(256) void dropout_mask_kernel(unsigned char* keep, da_abi::DropoutCfg cfg, int N, int stream) {
+  const int bh = blockIdx.y;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)N * N) return;
+  const unsigned q = (unsigned)(idx / N), k = (unsigned)(idx % N);
+  const unsigned word = dropout_word(cfg, 2u * bh + stream, (unsigned)N / 2, q >> 1, k >> 1);
+  keep[(size_t)bh * N * N + idx] = dropout_keep(word, q, k, cfg.threshold) ? 1 : 0;
+}
+
 inline size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 struct WsLayout {
@@ -102,7 +131,9 @@ WsLayout ws_layout(int BH, int N, int D) {
 template <class T>
 void fill_fwd(da_abi::FwdParamsT<T>& p, const void* q1, const void* q2, const void* k1, const void* k2,
               const void* v, const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
-              int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags, const Layouts& lay) {
+              int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags, const Layouts& lay,
+              const da_abi::DropoutCfg& drop) {
+  p.drop = drop;
   p.sqk = lay.qk; p.sv = lay.v; p.sy = lay.y;
   p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
   p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
@@ -121,7 +152,8 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
               void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
               void* ws_dx, void* ws_stat, void* ws_part, int n_part,
               int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags, unsigned stage_mask,
-              const Layouts& lay) {
+              const Layouts& lay, const da_abi::DropoutCfg& drop) {
+  p.drop = drop;
   p.sqk = lay.qk; p.sv = lay.v; p.sy = lay.y; p.sdy = lay.dy;
   p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
   p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
@@ -142,7 +174,7 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
 
 extern "C" {
 
-int diffattn_abi_version(void) { return 5; }
+int diffattn_abi_version(void) { return 6; }
 
 const char* diffattn_strerror(int code) {
   switch (code) {
@@ -154,6 +186,7 @@ const char* diffattn_strerror(int code) {
     case DIFFATTN_EINVAL_ALIGN: return "tensor pointers must be 16-byte aligned";
     case DIFFATTN_EINVAL_SCRATCH: return "problem too large for the built-in scratch of diffattn_backward_static (DIFFATTN_STATIC_SCRATCH_BYTES): use diffattn_backward with a caller workspace";
     case DIFFATTN_EINVAL_LAYOUT: return "bad strides in diffattn_layout: every stride must be a non-negative multiple of 8 elements and a row stride at least the row width";
+    case DIFFATTN_EINVAL_DROPOUT: return "dropout probability must lie in [0, 255/256]";
     case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL, DIFFATTN_BF16, DIFFATTN_LAMBDA_PER_HEAD)";
     default: break;
   }
@@ -166,13 +199,13 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
                      int B, int H, int N, int D, float sm_scale, float lambda_init, int flags,
                      void* stream) {
   return diffattn_forward_padded(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv,
-                                 B, H, N, N, D, sm_scale, lambda_init, flags, nullptr, stream);
+                                 B, H, N, N, D, sm_scale, lambda_init, flags, nullptr, nullptr, stream);
 }
 
 int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
                             const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
                             int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
-                            const diffattn_layout* layout, void* stream) {
+                            const diffattn_layout* layout, const diffattn_dropout* dropout, void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y) return DIFFATTN_EINVAL_NULL;
   if (flags & ~kKnownFlags) return DIFFATTN_EINVAL_FLAGS;
   if (int e = check_dims(B, H, N, D)) return e;
@@ -182,13 +215,15 @@ int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, cons
     return DIFFATTN_EINVAL_ALIGN;
   Layouts lay;
   if (int e = resolve_layout(layout, H, N, D, &lay)) return e;
+  da_abi::DropoutCfg drop;
+  if (int e = resolve_dropout(dropout, &drop)) return e;
   if (flags & DIFFATTN_BF16) {
     da_bf16::FwdParams p;
-    fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags, lay);
+    fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags, lay, drop);
     return (int)da_bf16::launch_fwd(p, D, (hipStream_t)stream);
   }
   FwdParams p;
-  fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags, lay);
+  fill_fwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, B * H, H, N, n_valid, sm_scale, lambda_init, flags, lay, drop);
   return (int)launch_fwd(p, D, (hipStream_t)stream);
 }
 
@@ -203,7 +238,8 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
                              void* dq1, void* dq2, void* dk1, void* dk2, void* dv, void* dlambda,
                              void* workspace, size_t workspace_bytes,
                              int B, int H, int N, int n_valid, int D, float sm_scale, float lambda_init, int flags,
-                             unsigned stage_mask, const diffattn_layout* layout, void* stream) {
+                             unsigned stage_mask, const diffattn_layout* layout, const diffattn_dropout* dropout,
+                             void* stream) {
   if (!q1 || !q2 || !k1 || !k2 || !v || !lambda_scale || !y || !u2 || !lse1 || !lse2 || !dy || !workspace)
     return DIFFATTN_EINVAL_NULL;
   // outputs are required by the stages that write them
@@ -219,6 +255,8 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
     if (!aligned16(q)) return DIFFATTN_EINVAL_ALIGN;
   Layouts lay;
   if (int e = resolve_layout(layout, H, N, D, &lay)) return e;
+  da_abi::DropoutCfg drop;
+  if (int e = resolve_dropout(dropout, &drop)) return e;
   const WsLayout w = ws_layout(B * H, N, D);
   if (workspace_bytes < w.total || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return DIFFATTN_EINVAL_WS;
   char* ws = (char*)workspace;
@@ -226,12 +264,12 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   if (flags & DIFFATTN_BF16) {
     da_bf16::BwdParams p;
     fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
-             ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask, lay);
+             ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask, lay, drop);
     return (int)da_bf16::launch_bwd(p, D, (hipStream_t)stream);
   }
   BwdParams p;
   fill_bwd(p, q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy, dq1, dq2, dk1, dk2, dv, dlambda,
-           ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask, lay);
+           ws + w.dx, ws + w.stat, ws + w.part, n_part, B * H, H, N, n_valid, sm_scale, lambda_init, flags, stage_mask, lay, drop);
   return (int)launch_bwd(p, D, (hipStream_t)stream);
 }
 
@@ -244,7 +282,7 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
                       void* stream) {
   return diffattn_backward_stages(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy,
                                   dq1, dq2, dk1, dk2, dv, dlambda, workspace, workspace_bytes,
-                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, nullptr, stream);
+                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, nullptr, nullptr, stream);
 }
 
 int diffattn_backward_static(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
@@ -263,7 +301,19 @@ int diffattn_backward_static(const void* q1, const void* q2, const void* k1, con
   // has to be cleared, whatever an earlier call left behind
   return diffattn_backward_stages(q1, q2, k1, k2, v, lambda_scale, y, u2, lse1, lse2, rinv, dy,
                                   dq1, dq2, dk1, dk2, dv, dlambda, ws, need,
-                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, nullptr, stream);
+                                  B, H, N, N, D, sm_scale, lambda_init, flags, DIFFATTN_STAGE_ALL, nullptr, nullptr, stream);
+}
+
+int diffattn_dropout_mask(unsigned char* keep, int B, int H, int N, int softmax_stream, const diffattn_dropout* dropout,
+                          void* stream) {
+  if (!keep || !dropout) return DIFFATTN_EINVAL_NULL;
+  if (B <= 0 || H <= 0 || N <= 0 || N % 2 != 0 || (long long)B * H > 65535 || (softmax_stream != 0 && softmax_stream != 1))
+    return DIFFATTN_EINVAL_DIM;
+  da_abi::DropoutCfg drop;
+  if (int e = resolve_dropout(dropout, &drop)) return e;
+  const dim3 grid((unsigned)(((size_t)N * N + 255) / 256), (unsigned)(B * H));
+  hipLaunchKernelGGL(dropout_mask_kernel, grid, dim3(256), 0, (hipStream_t)stream, keep, drop, N, softmax_stream);
+  return (int)hipGetLastError();
 }
 
 }  // extern "C"

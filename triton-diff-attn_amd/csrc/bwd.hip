@@ -151,7 +151,10 @@ struct DkvCfg {
 // K1, K2, V rows exceed the 512 registers of a lane, so the work is split in two launches:
 // MODE 1 computes dV only (scores S1, S2; no dP), MODE 2 computes dK1 and dK2 only.
 // CAUSAL: queries before the key block are skipped and the four sub-tiles on the diagonal are masked.
-template <int D, int MODE, bool CAUSAL>
+// DROP: dropout on both softmax maps, masks regenerated from the hash the forward used.  With the
+// keep mask m_t and c = 1/(1-p):  dS1 = A1 (c m1 dP - delta1),  dS2 = A2 (-lambda c m2 dP - delta2),
+// dV = c (m1 A1 - lambda m2 A2)^T dX; delta1, delta2 are the row dots with the dropped-out U1, U2.
+template <int D, int MODE, bool CAUSAL, bool DROP>
 __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_kernel(BwdParams p) {
   using C = DkvCfg<D>;
   constexpr int DV = C::DV, NW = C::NW, BK = C::BK, BQ = C::BQ;
@@ -276,13 +279,16 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     }
     return *reinterpret_cast<const h8*>(sQ1 + 2 * C::Q_TILE + swz_off<DV>(qs * 32 + j, 16 * (k >> 1) + 8 * g));
   };
+  // The dropout instantiations spill a few registers; there the products are issued as ordinary
+  // (compiler-visible) matrix instructions, so that the compiler places every wait state itself:
+  // with reloads of spilled fragments in front of them the opaque assembly form read stale operands.
   auto prod_mfma = [&](int k, h8 a, Scores& out) {
     if (!DO_K || (k & 1)) {
       const int t = DO_K ? (k >> 1) : k, ks = t >> 1;
-      if (t & 1) out.s2 = mfma32_bagpr(a, kf2[ks], out.s2);
-      else       out.s1 = mfma32_bagpr(a, kf1[ks], out.s1);
+      if (t & 1) out.s2 = DROP ? mfma32(a, kf2[ks], out.s2) : mfma32_bagpr(a, kf2[ks], out.s2);
+      else       out.s1 = DROP ? mfma32(a, kf1[ks], out.s1) : mfma32_bagpr(a, kf1[ks], out.s1);
     } else {
-      out.dp = mfma32_bagpr(a, vf[k >> 1], out.dp);
+      out.dp = DROP ? mfma32(a, vf[k >> 1], out.dp) : mfma32_bagpr(a, vf[k >> 1], out.dp);
     }
   };
   // Row statistics written by the preprocess kernel: 0: -lse1*log2e, 1: -lse2*log2e, 2: -delta1,
@@ -303,7 +309,8 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
 #pragma unroll
       for (int e = 0; e < 4; ++e) { out.s1[4 * r4 + e] = a[e]; out.s2[4 * r4 + e] = bq[e]; }
       if constexpr (DO_K) {
-        const f4v cq = stat4(buf, qs, 2, r4);
+        // with dropout the mask applies to dP alone, so -delta1 cannot ride in the accumulator
+        const f4v cq = DROP ? f4v{0.f, 0.f, 0.f, 0.f} : stat4(buf, qs, 2, r4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) out.dp[4 * r4 + e] = cq[e];
       }
@@ -312,14 +319,34 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   // Element-wise work of accumulator register r (query row 8*(r/4) + 4g + (r%4)), split in three
   // stages that are issued one product apart, so that no VALU instruction waits on the one
   // before it: (1) exponentials, (2) products, (3) fp16 packing of a pair of rows.
-  struct RowTmp { float p1[16], p2[16], u[16], ds1[16], ds2[16], pc[16]; };
+  struct RowTmp { float p1[16], p2[16], u[16], ds1[16], ds2[16], pc[16], a1[16], k1[16], k2[16]; unsigned w1, w2; };
   // `rel` (masked steps only) = key index minus the query index of register 0 of the sub-tile:
   // register r holds query 8*(r/4) + (r%4) relative to that, and a query before its key sees nothing
-  auto ew1 = [&](int r, const f4v& st3, const Scores& in, RowTmp& t, auto masked_tag, int rel) {
+  auto ew1 = [&](int r, const f4v& st3, const f4v& st2, const Scores& in, RowTmp& t, auto masked_tag, int rel, int qbase) {
     t.p1[r] = fast_exp2(in.s1[r]);
     t.p2[r] = fast_exp2(in.s2[r]);
     if constexpr (decltype(masked_tag)::value) {
       if (8 * (r / 4) + (r % 4) < rel) { t.p1[r] = 0.f; t.p2[r] = 0.f; }
+    }
+    if constexpr (DROP) {
+      // register r holds query qbase + 8*(r/4) + (r%4) of this lane's key; registers r, r+1 (r even)
+      // share the hash words of their 2x2 block, one word per softmax stream
+      const unsigned query = (unsigned)(qbase + 8 * (r / 4) + (r % 4));
+      if ((r & 1) == 0) {
+        t.w1 = dropout_word(p.drop, 2u * bh, (unsigned)p.N / 2, query >> 1, (unsigned)key >> 1);
+        t.w2 = dropout_word(p.drop, 2u * bh + 1, (unsigned)p.N / 2, query >> 1, (unsigned)key >> 1);
+      }
+      const bool keep1 = dropout_keep(t.w1, query, (unsigned)key, p.drop.threshold);
+      const bool keep2 = dropout_keep(t.w2, query, (unsigned)key, p.drop.threshold);
+      t.k1[r] = keep1 ? t.p1[r] : 0.f;
+      t.k2[r] = keep2 ? t.p2[r] : 0.f;
+      if constexpr (DO_K) {
+        const float dpc = p.drop.keep_scale * in.dp[r];
+        t.a1[r] = (keep1 ? dpc : 0.f) + st2[r % 4];                       // c m1 dP - delta1
+        // -delta2 = statistic 3 - lambda * statistic 2
+        t.u[r] = __builtin_fmaf(-lam, keep2 ? dpc : 0.f, __builtin_fmaf(-lam, st2[r % 4], st3[r % 4]));
+      }
+      return;
     }
     if constexpr (DO_K) {
       t.u[r] = __builtin_fmaf(-lam, in.dp[r], st3[r % 4]);
@@ -329,6 +356,14 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     }
   };
   auto ew2 = [&](int r, const Scores& in, RowTmp& t) {
+    if constexpr (DROP) {
+      if constexpr (DO_K) {
+        t.ds1[r] = t.p1[r] * t.a1[r];
+        t.ds2[r] = t.p2[r] * t.u[r];
+      }
+      if constexpr (DO_V) t.pc[r] = p.drop.keep_scale * __builtin_fmaf(-lam, t.k2[r], t.k1[r]);
+      return;
+    }
     if constexpr (DO_K) {
       t.ds1[r] = t.p1[r] * in.dp[r];
       t.ds2[r] = t.p2[r] * t.u[r];
@@ -346,8 +381,9 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     }
   };
   // slot s of the skewed schedule: stage 1 of row s, stage 2 of row s-1, stage 3 of the pair ending at row s-2
-  auto ew_slot = [&](int s, const f4v (&st)[4], const Scores& in, RowTmp& t, Packed& out, auto masked_tag, int rel) {
-    if (s < 16) ew1(s, st[s / 4], in, t, masked_tag, rel);
+  auto ew_slot = [&](int s, const f4v (&st)[4], const f4v (&st2)[4], const Scores& in, RowTmp& t, Packed& out, auto masked_tag,
+                     int rel, int qbase) {
+    if (s < 16) ew1(s, st[s / 4], st2[s / 4], in, t, masked_tag, rel, qbase);
     if (s >= 1 && s - 1 < 16) ew2(s - 1, in, t);
     if (s >= 2 && s - 2 < 16 && ((s - 2) & 1)) ew3(s - 2, t, out);
   };
@@ -396,7 +432,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   static_assert(NPROD % 16 == 0 || 16 % NPROD == 0, "rows are spread evenly over the products");
   constexpr int AHEAD = 3;                     // B fragments requested ahead of their product
   auto fused = [&](int bufn, int qsn, Scores& s_nxt, int bufc, int qsc, const Scores& s_cur, Packed& pk,
-                   int bufp, int qsp, int tile_next, int buf_next, bool fetch, auto masked_tag, int rel) {
+                   int bufp, int qsp, int tile_next, int buf_next, bool fetch, auto masked_tag, int rel, int qbase) {
     constexpr int NSLOT = 18;                  // 16 rows + 2 slots of pipeline drain
     constexpr int LEAD = 2;                    // slots run before the first product
     // rows 0..7 are packed by slot 9, which must precede the first product that reads them
@@ -406,17 +442,21 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
       return (ja < NACC / 2) ? acc_frag(bufp, qsp, m) : acc_frag(bufc, qsc, m);
     };
     h8 a[NPROD], bf[NACC];
-    f4v st[4];
+    f4v st[4], st2[4];
     RowTmp tmp;
     init_scores(bufn, qsn, s_nxt);
 #pragma unroll
     for (int k = 0; k < DEPTH; ++k) a[k] = prod_frag(bufn, qsn, k);
     if constexpr (DO_K) st[0] = stat4(bufc, qsc, 3, 0);
+    if constexpr (DO_K && DROP) {
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) st2[r4] = stat4(bufc, qsc, 2, r4);
+    }
 #pragma unroll
     for (int k = 0; k < AHEAD; ++k) bf[k] = bfrag(k);
     // the first slots run while the initial accumulator values and the first fragments arrive
 #pragma unroll
-    for (int s = 0; s < LEAD; ++s) ew_slot(s, st, s_cur, tmp, pk, masked_tag, rel);
+    for (int s = 0; s < LEAD; ++s) ew_slot(s, st, st2, s_cur, tmp, pk, masked_tag, rel, qbase);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int k = 0; k < NPROD; ++k) {
@@ -431,7 +471,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
       // slots LEAD .. NSLOT-1 spread over the products
       const int s0 = LEAD + (NSLOT - LEAD) * k / NPROD, s1 = LEAD + (NSLOT - LEAD) * (k + 1) / NPROD;
 #pragma unroll
-      for (int s = s0; s < s1; ++s) ew_slot(s, st, s_cur, tmp, pk, masked_tag, rel);
+      for (int s = s0; s < s1; ++s) ew_slot(s, st, st2, s_cur, tmp, pk, masked_tag, rel, qbase);
       __builtin_amdgcn_sched_barrier(0);
     }
     // the next step's VALU reads these results right away
@@ -455,7 +495,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     // past the end the last sub-tile is scored again and the result is never used; before the
     // start the all-zero upper operand half is accumulated against the first tile
     fused(buf_of(tn), more ? SUBN : SUBC, s_nxt, buf_of(tc), SUBC, s_cur, pk,
-          buf_of(tp), (i > i0) ? SUBP : 0, tl, buf_of(tn + 1), opens, masked_tag, key - 32 * i - 4 * g);
+          buf_of(tp), (i > i0) ? SUBP : 0, tl, buf_of(tn + 1), opens, masked_tag, key - 32 * i - 4 * g, 32 * i + 4 * g);
   };
 
   // prologue: the first tile, then start fetching the second; scores of the first sub-tile
@@ -549,7 +589,8 @@ struct DqCfg {
 // MASK: 0 none; 1 causal (key <= query); 2 the last keys of the sequence are padding (key < n_keys).
 // A padded key has a zero K row, but its recomputed "probability" exp(0 - lse) is not small when a
 // row's logsumexp is negative, and its dS can overflow fp16: it must be masked, not multiplied by 0.
-template <int D, int NWAVES, int MASK>
+// DROP: dropout on both softmax maps, as in bwd_dkdv_kernel.
+template <int D, int NWAVES, int MASK, bool DROP>
 __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_waves_per_eu(DqCfg<D, NWAVES>::OCC, DqCfg<D, NWAVES>::OCC))) void bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<D, NWAVES>;
   constexpr bool CAUSAL = (MASK == 1), PADDED = (MASK == 2);
@@ -709,13 +750,30 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       }
       __builtin_amdgcn_sched_barrier(0);
       h8 b1[2], b2[2];
+      unsigned w1 = 0, w2 = 0;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float p1 = fast_exp2(s1[r] + nl1);
         const float p2 = fast_exp2(s2[r] + nl2);
-        const float dpc = dp[r] + de1;                  // statistic 2 is -delta1
-        b1[r / 8][r % 8] = (half_t)(p1 * dpc);
-        b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dpc, de2));   // statistic 3 is -(lambda*delta1 + delta2)
+        if constexpr (DROP) {
+          // register r holds key kq + 8*(r/4) + (r%4) of this lane's query; registers r, r+1 (r even)
+          // share the hash words of their 2x2 block
+          const unsigned query = (unsigned)(qt * BM + wave * 32 + j);
+          const unsigned kq = (unsigned)(t * BN + ksub * 32 + 4 * g + 8 * (r / 4) + (r % 4));
+          if ((r & 1) == 0) {
+            w1 = dropout_word(p.drop, 2u * bh, (unsigned)p.N / 2, query >> 1, kq >> 1);
+            w2 = dropout_word(p.drop, 2u * bh + 1, (unsigned)p.N / 2, query >> 1, kq >> 1);
+          }
+          const float dpk = p.drop.keep_scale * dp[r];
+          const float d1 = dropout_keep(w1, query, kq, p.drop.threshold) ? dpk : 0.f;
+          const float d2 = dropout_keep(w2, query, kq, p.drop.threshold) ? dpk : 0.f;
+          b1[r / 8][r % 8] = (half_t)(p1 * (d1 + de1));                                             // c m1 dP - delta1
+          b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, d2, __builtin_fmaf(-lam, de1, de2)));   // -lambda c m2 dP - delta2
+        } else {
+          const float dpc = dp[r] + de1;                  // statistic 2 is -delta1
+          b1[r / 8][r % 8] = (half_t)(p1 * dpc);
+          b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dpc, de2));   // statistic 3 is -(lambda*delta1 + delta2)
+        }
       }
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk)
@@ -773,15 +831,22 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
   }
   if (p.stages & 4u) {
     const dim3 grid(p.BH * (p.N / DkvCfg<D>::BK)), block(DkvCfg<D>::NT);
+    auto launch_mode = [&](auto mode_tag) {
+      constexpr int M = decltype(mode_tag)::value;
+      if (p.drop.threshold) {
+        if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, true, true>), grid, block, 0, stream, p);
+        else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, false, true>), grid, block, 0, stream, p);
+      } else {
+        if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, true, false>), grid, block, 0, stream, p);
+        else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, false, false>), grid, block, 0, stream, p);
+      }
+    };
     if constexpr (D == 128) {
-      if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, 1, true>), grid, block, 0, stream, p);
-      else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, 1, false>), grid, block, 0, stream, p);
+      launch_mode(std::integral_constant<int, 1>{});
       if ((e = hipGetLastError()) != hipSuccess) return e;
-      if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, 2, true>), grid, block, 0, stream, p);
-      else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, 2, false>), grid, block, 0, stream, p);
+      launch_mode(std::integral_constant<int, 2>{});
     } else {
-      if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, 0, true>), grid, block, 0, stream, p);
-      else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, 0, false>), grid, block, 0, stream, p);
+      launch_mode(std::integral_constant<int, 0>{});
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
@@ -792,20 +857,28 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
     // in twice as many, half as long workgroups.
     constexpr int kNumCU = 256;
     bool wide = false;
+    auto launch_dq = [&](auto nw_tag, dim3 grid, dim3 block) {
+      constexpr int NWV = decltype(nw_tag)::value;
+      if (p.drop.threshold) {
+        if (p.causal)            hipLaunchKernelGGL((bwd_dq_kernel<D, NWV, 1, true>), grid, block, 0, stream, p);
+        else if (p.n_keys < p.N) hipLaunchKernelGGL((bwd_dq_kernel<D, NWV, 2, true>), grid, block, 0, stream, p);
+        else                     hipLaunchKernelGGL((bwd_dq_kernel<D, NWV, 0, true>), grid, block, 0, stream, p);
+      } else {
+        if (p.causal)            hipLaunchKernelGGL((bwd_dq_kernel<D, NWV, 1, false>), grid, block, 0, stream, p);
+        else if (p.n_keys < p.N) hipLaunchKernelGGL((bwd_dq_kernel<D, NWV, 2, false>), grid, block, 0, stream, p);
+        else                     hipLaunchKernelGGL((bwd_dq_kernel<D, NWV, 0, false>), grid, block, 0, stream, p);
+      }
+    };
     if constexpr (D != 128) {
       if (p.N % 256 == 0 && (long long)p.BH * (p.N / 128) > kNumCU) {
         wide = true;
         const dim3 grid(p.BH * (p.N / 256)), block(512);
-        if (p.causal)            hipLaunchKernelGGL((bwd_dq_kernel<D, 8, 1>), grid, block, 0, stream, p);
-        else if (p.n_keys < p.N) hipLaunchKernelGGL((bwd_dq_kernel<D, 8, 2>), grid, block, 0, stream, p);
-        else                     hipLaunchKernelGGL((bwd_dq_kernel<D, 8, 0>), grid, block, 0, stream, p);
+        launch_dq(std::integral_constant<int, 8>{}, grid, block);
       }
     }
     if (!wide) {
       const dim3 grid(p.BH * (p.N / 128)), block(256);
-      if (p.causal)            hipLaunchKernelGGL((bwd_dq_kernel<D, 4, 1>), grid, block, 0, stream, p);
-      else if (p.n_keys < p.N) hipLaunchKernelGGL((bwd_dq_kernel<D, 4, 2>), grid, block, 0, stream, p);
-      else                     hipLaunchKernelGGL((bwd_dq_kernel<D, 4, 0>), grid, block, 0, stream, p);
+      launch_dq(std::integral_constant<int, 4>{}, grid, block);
     }
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }

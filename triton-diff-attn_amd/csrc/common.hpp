@@ -23,6 +23,15 @@
 #define DA_MFMA_32x32x16 "v_mfma_f32_32x32x16_f16"
 #endif
 
+namespace da_abi {
+// dropout parameters as the kernels see them (one definition for both builds)
+struct DropoutCfg {
+  unsigned seed_lo, seed_hi;
+  unsigned threshold;           // 0 (no dropout) .. 255: a pair is kept iff its random byte >= threshold
+  float keep_scale;             // 1 / (1 - threshold/256)
+};
+}  // namespace da_abi
+
 namespace DA_NS {
 
 #ifdef DA_BF16
@@ -227,6 +236,29 @@ __device__ __forceinline__ void wait_async_tiles_except(int newest) {
     case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
     default: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
   }
+}
+
+// ---- dropout ------------------------------------------------------------------------------------
+// Keep/drop decisions come from a counter-based hash, so that forward, both backward kernels and the
+// mask dump agree without storing anything: one 32-bit word per 2x2 block of (query, key) pairs,
+// keyed on (seed, softmax stream, batch*head unit, query/2, key/2); the pair (q, k) owns byte
+// 2*(q&1) + (k&1) of the word and is kept iff that byte >= threshold, threshold = round(256 p).
+using da_abi::DropoutCfg;
+
+__device__ __forceinline__ unsigned dropout_word(const DropoutCfg& c, unsigned stream_unit, unsigned half_n, unsigned qh, unsigned kh) {
+  unsigned h = (qh * half_n + kh) ^ c.seed_lo;
+  h *= 0x9E3779B1u;
+  h ^= h >> 15;
+  h += (stream_unit * 0x85EBCA77u) ^ c.seed_hi;
+  h *= 0xC2B2AE3Du;
+  h ^= h >> 13;
+  h *= 0x27D4EB2Fu;
+  h ^= h >> 16;
+  return h;
+}
+// keep decision of pair (q, k) from the word of its 2x2 block
+__device__ __forceinline__ bool dropout_keep(unsigned word, unsigned q, unsigned k, unsigned threshold) {
+  return ((word >> (8 * (2 * (q & 1) + (k & 1)))) & 0xffu) >= threshold;
 }
 
 // Workgroup id -> logical tile id such that consecutive logical ids land on the same XCD

@@ -40,7 +40,10 @@ constexpr float kRescaleThreshold = 8.0f;   // log2 units: probabilities stay be
 
 // MASK: 0 none; 1 causal (key <= query); 2 the last keys of the sequence are padding (key < n_keys).
 // With the causal mask the padding needs no extra test: a padded key lies after every real query.
-template <int D, bool RMS, int MASK>
+// DROP: dropout on both softmax maps (not in the reference, which lists it as missing,
+// src/kernel.py:4): a dropped probability still counts in its row's sum but not in P*V, and the
+// kept ones are scaled by 1/(1-p) -- in the epilogue, together with 1/l.
+template <int D, bool RMS, int MASK, bool DROP>
 __global__ __launch_bounds__(FwdCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::OCC, FwdCfg<D>::OCC)))
 void fwd_kernel(FwdParams p) {
   using C = FwdCfg<D>;
@@ -274,7 +277,16 @@ void fwd_kernel(FwdParams p) {
           e2[0] = (half_t)fast_exp2(s_cur[qs][kt][r]);
           e2[1] = (half_t)fast_exp2(s_cur[qs][kt][r + 1]);
           rs = add_pair(e2, rs);   // row sum of the rounded probabilities
-          pw[qs][kt * 2 + r / 8][(r % 8) / 2] = __builtin_bit_cast(unsigned, e2);
+          unsigned w2 = __builtin_bit_cast(unsigned, e2);
+          if constexpr (DROP) {
+            // registers r, r+1 hold the keys key, key+1 (key even) of this lane's query
+            const unsigned query = (unsigned)(qrow0 + 32 * qs);
+            const unsigned key = (unsigned)(t * BN + kt * 32 + 8 * (r / 4) + 4 * g + (r % 4));
+            const unsigned word = dropout_word(p.drop, 2u * bh + st, (unsigned)p.N / 2, query >> 1, key >> 1);
+            w2 &= (dropout_keep(word, query, key, p.drop.threshold) ? 0x0000ffffu : 0u) |
+                  (dropout_keep(word, query, key + 1, p.drop.threshold) ? 0xffff0000u : 0u);
+          }
+          pw[qs][kt * 2 + r / 8][(r % 8) / 2] = w2;
         }
       l[qs] += rs;
     }
@@ -350,7 +362,7 @@ void fwd_kernel(FwdParams p) {
 
   static_assert(QS == 1, "the epilogue stages one 32-row block per wave");
   const float lsum = pair_sum(l[0]);
-  const float inv = 1.0f / lsum;
+  const float inv = (DROP ? p.drop.keep_scale : 1.0f) / lsum;
   const size_t row = (size_t)bh * p.N + qrow0;
   const size_t wave_row0 = (size_t)bh * p.N + qt * BM + qw * 32;
   {
@@ -390,23 +402,27 @@ void fwd_kernel(FwdParams p) {
   }
 }
 
-template <int D, bool RMS>
+template <int D, bool RMS, bool DROP>
 static void launch_fwd_c(const FwdParams& p, dim3 grid, dim3 block, hipStream_t stream) {
   if (p.causal)
-    hipLaunchKernelGGL((fwd_kernel<D, RMS, 1>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, 1, DROP>), grid, block, 0, stream, p);
   else if (p.n_keys < p.N)
-    hipLaunchKernelGGL((fwd_kernel<D, RMS, 2>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, 2, DROP>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((fwd_kernel<D, RMS, 0>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, 0, DROP>), grid, block, 0, stream, p);
 }
 
 template <int D>
 static hipError_t launch_fwd_t(const FwdParams& p, hipStream_t stream) {
   dim3 grid(p.BH * (p.N / FwdCfg<D>::BM)), block(FwdCfg<D>::NT);
-  if (p.rms_norm)
-    launch_fwd_c<D, true>(p, grid, block, stream);
-  else
-    launch_fwd_c<D, false>(p, grid, block, stream);
+  const bool drop = p.drop.threshold != 0;
+  if (p.rms_norm) {
+    if (drop) launch_fwd_c<D, true, true>(p, grid, block, stream);
+    else      launch_fwd_c<D, true, false>(p, grid, block, stream);
+  } else {
+    if (drop) launch_fwd_c<D, false, true>(p, grid, block, stream);
+    else      launch_fwd_c<D, false, false>(p, grid, block, stream);
+  }
   return hipGetLastError();
 }
 

@@ -25,6 +25,7 @@ struct FwdParamsT {
   int H;                        // heads per batch entry: unit bh belongs to head bh % H
   int lambda_stride;            // 0: lambda_scale[0] for every head; 1: lambda_scale[head]
   Strides sqk, sv, sy;          // layouts of q1,q2,k1,k2 / v / y; u2 and the row statistics are dense
+  DropoutCfg drop;               // threshold 0: no dropout
 };
 
 template <class T>
@@ -50,6 +51,7 @@ struct BwdParamsT {
   int H;                        // heads per batch entry: unit bh belongs to head bh % H
   int lambda_stride;            // 0: one lambda; 1: one per head
   Strides sqk, sv, sy, sdy;     // layouts of q1,q2,k1,k2 / v / y / dy; everything else is dense
+  DropoutCfg drop;               // threshold 0: no dropout
 };
 
 // lambda of the (batch, head) unit bh

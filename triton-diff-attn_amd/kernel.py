@@ -1,8 +1,9 @@
 """Autograd wiring of the MI355X differential-attention kernels.
 
 Host-side counterpart of the reference's `_diff_attention` (src/kernel.py:461-575): same class
-name, same `apply` argument order, same 9-slot gradient tuple (a tenth, optional argument `causal`
--- masking is a feature the reference lists as missing, src/kernel.py:4 -- adds a tenth slot).  The work itself is done by the
+name, same `apply` argument order, same 9-slot gradient tuple (the optional arguments `causal`,
+`dropout_p` and `dropout_seed` -- masking and dropout are features the reference lists as missing,
+src/kernel.py:4 -- add a slot each).  The work itself is done by the
 hand-written HIP kernels in libdiffattn.so, reached through its C ABI; if the library is missing
 the call raises -- there is no other path.
 """
@@ -96,8 +97,14 @@ def _ptr(t):
 class _diff_attention(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, Q1, Q2, K1, K2, V, SM_SCALE, LAMBDA_SCALE, LAMBDA_INIT, rms_norm=False, causal=False):
+    def forward(ctx, Q1, Q2, K1, K2, V, SM_SCALE, LAMBDA_SCALE, LAMBDA_INIT, rms_norm=False, causal=False,
+                dropout_p=0.0, dropout_seed=0):
         B, H, N, D = _check_inputs(Q1, Q2, K1, K2, V)
+        dropout_p = float(dropout_p)
+        if not 0.0 <= dropout_p <= 255 / 256:
+            raise ValueError("dropout_p must lie in [0, 255/256] (got %r)" % dropout_p)
+        # the same struct goes to the backward: the masks are a function of (seed, position) only
+        dropout = _native.Dropout(dropout_p, int(dropout_seed) & 0xFFFFFFFFFFFFFFFF) if dropout_p > 0 else None
         lib = _native.lib()
         dev = Q1.device
         # The kernels work on multiples of 128 rows (like the reference's, src/kernel.py:527).  Other
@@ -139,12 +146,12 @@ class _diff_attention(torch.autograd.Function):
                 rc = lib.diffattn_forward_padded(
                     q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
                     lam.data_ptr(), y.data_ptr(), _ptr(u2), _ptr(lse1), _ptr(lse2), _ptr(rinv),
-                    B, H, n_pad, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, layout, _current_stream(dev))
+                    B, H, n_pad, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, layout, dropout, _current_stream(dev))
         else:
             rc = lib.diffattn_forward_padded(
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
                 lam.data_ptr(), y.data_ptr(), _ptr(u2), _ptr(lse1), _ptr(lse2), _ptr(rinv),
-                B, H, n_pad, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, layout, _current_stream(dev))
+                B, H, n_pad, N, D, float(SM_SCALE), float(LAMBDA_INIT), flags, layout, dropout, _current_stream(dev))
         _native.check(rc)
 
         if differentiable:
@@ -153,6 +160,7 @@ class _diff_attention(torch.autograd.Function):
         ctx.LAMBDA_INIT = float(LAMBDA_INIT)
         ctx.FLAGS = flags
         ctx.N_VALID = N
+        ctx.DROPOUT = dropout
         ctx.lambda_meta = (LAMBDA_SCALE.dtype, LAMBDA_SCALE.shape) if torch.is_tensor(LAMBDA_SCALE) else None
         return y if n_pad == N else y[:, :, :N].contiguous()
 
@@ -198,7 +206,7 @@ class _diff_attention(torch.autograd.Function):
                 y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv), dO.data_ptr(),
                 _ptr(dq1), _ptr(dq2), _ptr(dk1), _ptr(dk2), _ptr(dv), _ptr(dlam),
                 ws.data_ptr(), ws_bytes, B, H, N, n_valid, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stages,
-                layout, _current_stream(dev))
+                layout, ctx.DROPOUT, _current_stream(dev))
 
         if dev.index is not None and dev.index != torch._C._cuda_getDevice():
             with torch.cuda.device(dev):
@@ -214,5 +222,5 @@ class _diff_attention(torch.autograd.Function):
         if n_valid != N:
             dq1, dq2, dk1, dk2, dv = (None if t is None else t[:, :, :n_valid].contiguous()
                                       for t in (dq1, dq2, dk1, dk2, dv))
-        # one slot per forward argument: nine, or ten when `causal` was passed
+        # one slot per forward argument: nine, or more when causal / dropout arguments were passed
         return (dq1, dq2, dk1, dk2, dv, None, dlambda) + (None,) * (len(ctx.needs_input_grad) - 7)

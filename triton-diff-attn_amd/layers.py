@@ -19,6 +19,8 @@ def MultiheadDiffAttnKernel(
     lambda_init: float = 0.8,
     rms_norm: bool = False,
     causal: bool = False,
+    dropout_p: float = 0.0,
+    dropout_seed=None,
 ):
     """(softmax(q1 k1^T / sqrt(d)) - lambda_scale * softmax(q2 k2^T / sqrt(d))) v, optionally followed
     by a per-row RMSNorm over the 2d output features and a (1 - lambda_init) scale.
@@ -27,10 +29,18 @@ def MultiheadDiffAttnKernel(
     (a python float is accepted too; a tensor of H elements gives every head its own lambda, which
     the reference does not have).  Returns [B, H, N, 2d] fp16 with autograd support for the
     five tensors and lambda_scale.  `causal` (not in the reference, which lists masking as missing,
-    src/kernel.py:4) lets query i attend to keys 0..i only.
+    src/kernel.py:4) lets query i attend to keys 0..i only.  `dropout_p` (likewise missing in the
+    reference) drops every entry of each of the two softmax maps independently with that
+    probability, in steps of 1/256, and scales the kept ones by 1/(1-p); the masks are a function of
+    `dropout_seed` (drawn from torch's default generator when None) and the position.
     """
     head_dim = q1.size(-1)
     sm_scale = 1 / math.sqrt(head_dim)
+    if dropout_p:
+        if dropout_seed is None:
+            dropout_seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+        return _diff_attention.apply(q1, q2, k1, k2, v, sm_scale, lambda_scale, lambda_init, rms_norm, bool(causal),
+                                     float(dropout_p), int(dropout_seed))
     if causal:
         return _diff_attention.apply(q1, q2, k1, k2, v, sm_scale, lambda_scale, lambda_init, rms_norm, True)
     return _diff_attention.apply(q1, q2, k1, k2, v, sm_scale, lambda_scale, lambda_init, rms_norm)

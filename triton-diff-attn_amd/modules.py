@@ -4,7 +4,8 @@ The reference stops at the functional operator (src/layers.py:10-26); its kernel
 the Differential Transformer paper (src/kernel.py:1) for the layer around it.  This module is that
 layer: input projections, the re-parametrised lambda, the fused operator with its per-head RMSNorm
 and (1 - lambda_init) scale, a learnable per-feature gain on the normalised heads, and the output
-projection.  Attention is bidirectional unless `causal=True`.
+projection.  Attention is bidirectional unless `causal=True`; `attention_dropout` drops entries of
+the two softmax maps while the module is in training mode.
 
   x [B, N, E]  ->  q, k [B, 2H, N, d],  v [B, H, N, 2d]      (E = 2 * H * d)
   lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + lambda_init       (one scalar per layer, or one per
@@ -27,7 +28,8 @@ def lambda_init_for_depth(depth: int) -> float:
 
 class DiffAttn(nn.Module):
     def __init__(self, embed_dim: int, num_heads: int, depth: int = 0, attention=MultiheadDiffAttnKernel,
-                 causal: bool = False, per_head_lambda: bool = False, device=None, dtype=torch.float16):
+                 causal: bool = False, per_head_lambda: bool = False, attention_dropout: float = 0.0,
+                 device=None, dtype=torch.float16):
         super().__init__()
         if embed_dim % (2 * num_heads) != 0:
             raise ValueError("embed_dim must be divisible by 2 * num_heads")
@@ -37,6 +39,7 @@ class DiffAttn(nn.Module):
         self.lambda_init = lambda_init_for_depth(depth)
         self.attention = attention
         self.causal = causal
+        self.attention_dropout = float(attention_dropout)     # on both softmax maps, in training mode only
         kw = dict(device=device, dtype=dtype)
         self.q_proj = nn.Linear(embed_dim, embed_dim, bias=False, **kw)
         self.k_proj = nn.Linear(embed_dim, embed_dim, bias=False, **kw)
@@ -67,6 +70,7 @@ class DiffAttn(nn.Module):
         # views of the projection outputs: the operator reads them through their strides and returns the
         # heads in v's [B,N,H,2d] memory layout, so neither side of it copies
         heads = self.attention(q[0], q[1], k[0], k[1], v, lambda_scale=lam, lambda_init=self.lambda_init, rms_norm=True,
-                               **({"causal": True} if self.causal else {}))
+                               **({"causal": True} if self.causal else {}),
+                               **({"dropout_p": self.attention_dropout} if self.training and self.attention_dropout else {}))
         heads = heads * self.head_gain
         return self.out_proj(heads.transpose(1, 2).reshape(B, N, E))
