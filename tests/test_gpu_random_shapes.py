@@ -57,3 +57,48 @@ def test_random_problem_matches_oracle(seed):
     # d(lambda) sums many terms of either sign; its error is measured against the gradient scale of the run
     denom = max(ref[6].abs().max().item(), 1e-3 * sum(r.abs().max().item() for r in ref[1:6]) * N ** 0.5)
     assert (lam_dev.grad.float().cpu() - ref[6]).abs().max().item() <= (3 * g_tol) * denom
+
+
+@pytest.mark.parametrize("seed", range(100, 112))
+def test_random_problem_with_dropout_and_strided_tensors(seed):
+    """As above, with dropout drawn in and, for every other seed, the tensors living in [B,N,H,C] buffers."""
+    from layers import MultiheadDiffAttnKernel
+    from test_gpu_dropout import kernel_masks
+
+    cfg = draw(seed)
+    rnd = random.Random(7 * seed)
+    p = rnd.choice([0.1, 0.3, 0.5])
+    token_major = seed % 2 == 0
+    print("case", cfg, dict(p=p, token_major=token_major), flush=True)
+    B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
+    dt = torch.bfloat16 if cfg["bf16"] else torch.float16
+    g = torch.Generator().manual_seed(2000 + seed)
+    mk = lambda d: torch.randn(B, H, N, d, generator=g).to(dt)
+    q1, q2, k1, k2, v, dy = mk(D), mk(D), mk(D), mk(D), mk(2 * D), mk(2 * D)
+    n_lam = H if cfg["per_head"] else 1
+    lam = (torch.rand(n_lam, generator=g) * 1.6 - 0.6).to(dt)
+
+    place = (lambda t: t.cuda().transpose(1, 2).contiguous().transpose(1, 2)) if token_major else (lambda t: t.cuda())
+    leaves = [place(t).requires_grad_(True) for t in (q1, q2, k1, k2, v)]
+    lam_dev = lam.cuda().requires_grad_(True)
+    y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam_dev, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"],
+                                causal=cfg["causal"], dropout_p=p, dropout_seed=seed)
+    y.backward(place(dy))
+    torch.cuda.synchronize()
+
+    n_pad = -(-N // 128) * 128
+    m1, m2 = (m[:, :, :N, :N] for m in kernel_masks(B, H, n_pad, p, seed))
+    ref = orc.forward_backward(q1, q2, k1, k2, v, lam, dy, cfg["lambda_init"], cfg["rms"], causal=cfg["causal"],
+                               keep1=m1, keep2=m2, dropout_p=round(p * 256) / 256)
+    y_tol, g_tol = (6e-2, 8e-2) if cfg["bf16"] else (Y_ATOL, GRAD_RTOL)
+    # a row whose kept weights happen to be few is scaled by 1/(1-p): allow for that factor
+    y_tol, g_tol = y_tol / (1 - p), g_tol
+    assert torch.isfinite(y).all() and max_abs(y.detach(), ref[0]) <= y_tol
+    for name, t, want in zip(("dq1", "dq2", "dk1", "dk2", "dv"), leaves, ref[1:6]):
+        scale = want.abs().max().item()
+        if scale == 0.0:
+            assert t.grad.float().abs().max().item() <= 1e-3, name
+        else:
+            assert rel_to_max(t.grad, want) <= g_tol, name
+    denom = max(ref[6].abs().max().item(), 1e-3 * sum(r.abs().max().item() for r in ref[1:6]) * N ** 0.5)
+    assert (lam_dev.grad.float().cpu() - ref[6]).abs().max().item() <= (3 * g_tol) * denom

@@ -265,7 +265,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   struct Scores { f16v s1, s2, dp; };
   struct Packed { h8 pc[2], d1[2], d2[2]; };   // A operands of the dV / dK1 / dK2 products
   constexpr int NPROD = 2 * NKS + (DO_K ? NKV : 0);   // score products per sub-tile (dP is needed for dK only)
-  constexpr int DEPTH = 3;                     // A fragments requested ahead of their product
+  constexpr int DEPTH = DROP ? 1 : 3;          // A fragments requested ahead of their product (dropout: registers are short)
 
   // Product k of a sub-tile: even k is k-step k/2 of dP, odd k alternates k-steps of S1 and S2, so
   // the three accumulation chains advance together; without dP (MODE 1) S1 and S2 alternate.
@@ -430,7 +430,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   // of the step and read during the second, its upper half is written during the second half and
   // read during the first half of the next step.
   static_assert(NPROD % 16 == 0 || 16 % NPROD == 0, "rows are spread evenly over the products");
-  constexpr int AHEAD = 3;                     // B fragments requested ahead of their product
+  constexpr int AHEAD = DROP ? 1 : 3;          // B fragments requested ahead of their product
   auto fused = [&](int bufn, int qsn, Scores& s_nxt, int bufc, int qsc, const Scores& s_cur, Packed& pk,
                    int bufp, int qsp, int tile_next, int buf_next, bool fetch, auto masked_tag, int rel, int qbase) {
     constexpr int NSLOT = 18;                  // 16 rows + 2 slots of pipeline drain
@@ -736,17 +736,21 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       // The transposed K fragments of the dQ products do not depend on the element-wise work: they
       // are requested before it and arrive while it runs.  (Left to itself the compiler requests
       // each one right in front of its product and waits out the LDS latency eight times.)
+      // (The dropout instantiations need the registers for the mask arithmetic and read each
+      // fragment in front of its product instead.)
       h8 tk1[2][NDT], tk2[2][NDT];
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
+      auto read_tk = [&](int kk, int tt) {
         const int rbase = ksub * 32 + 16 * kk + tr_row;
+        tk1[kk][tt] = join(lds_read_tr(sK1 + swz_off<D>(rbase, 32 * tt + tr_col)),
+                           lds_read_tr(sK1 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
+        tk2[kk][tt] = join(lds_read_tr(sK2 + swz_off<D>(rbase, 32 * tt + tr_col)),
+                           lds_read_tr(sK2 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
+      };
+      if constexpr (!DROP) {
 #pragma unroll
-        for (int tt = 0; tt < NDT; ++tt) {
-          tk1[kk][tt] = join(lds_read_tr(sK1 + swz_off<D>(rbase, 32 * tt + tr_col)),
-                             lds_read_tr(sK1 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
-          tk2[kk][tt] = join(lds_read_tr(sK2 + swz_off<D>(rbase, 32 * tt + tr_col)),
-                             lds_read_tr(sK2 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
-        }
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+          for (int tt = 0; tt < NDT; ++tt) read_tk(kk, tt);
       }
       __builtin_amdgcn_sched_barrier(0);
       h8 b1[2], b2[2];
@@ -779,6 +783,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
         for (int tt = 0; tt < NDT; ++tt) {
+          if constexpr (DROP) read_tk(kk, tt);
           dq1[tt] = mfma32(tk1[kk][tt], b1[kk], dq1[tt]);
           dq2[tt] = mfma32(tk2[kk][tt], b2[kk], dq2[tt]);
         }

@@ -262,6 +262,9 @@ void fwd_kernel(FwdParams p) {
     // tile run on the matrix unit while the exponentials run on the VALU.
     load_k2(tk, kb0);
     scores(ka, s_nxt);
+    // dropout: the mask arithmetic needs the registers of the K fragments, so the score product is
+    // issued in full before the exponentials instead of between them
+    if constexpr (DROP) __builtin_amdgcn_sched_barrier(0);
 
     // P^T as B operands: pb[kk] covers keys 16kk..16kk+15 (accumulator order).  Built from the packed
     // pairs as 32-bit words, so that each pair is converted once, for the row sum and the operand alike.
@@ -295,7 +298,7 @@ void fwd_kernel(FwdParams p) {
     // 3 are 1.3 % faster than the single product the compiler picks by itself, 5 and 7 are not)
     const half_t* sV = sVbuf + vb0 * C::V_TILE;
     constexpr int NPV = NKK * NOT;
-    constexpr int PD = 3;
+    constexpr int PD = DROP ? 1 : 3;           // dropout: registers are short
     auto vt_frag = [&](int i) {
       const int kk = i / NOT, tt = i % NOT;
       return join(lds_read_tr(sV + swz_off<DV>(16 * kk + tr_row, 32 * tt + tr_col)),
