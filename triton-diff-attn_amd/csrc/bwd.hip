@@ -796,12 +796,16 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
     bnext = (bnext == 2) ? 0 : bnext + 1;
   }
   wait_async_tiles();
+  __syncthreads();      // the tile memory is reused below; other waves may still have been reading it
 
   // dQ^T tile tt: this lane's column is its query; register r = feature 32*tt + 8*(r/4) + 4g + (r%4).
   // The accumulated sums carry log2(e) from the pre-scaled Q only inside the probabilities, so the
-  // remaining factor is the plain softmax scale.
-  half_t* o1 = p.dq1 + qrow * D;
-  half_t* o2 = p.dq2 + qrow * D;
+  // remaining factor is the plain softmax scale.  Each wave stages its 32 rows of dQ1 and dQ2 in the
+  // now idle tile memory (8 bytes per lane, row stride D+8 halfs) and reads them back row by row, so
+  // that the global stores are whole 16-byte chunks of consecutive rows.
+  constexpr int SROW = D + 8;
+  static_assert(NW * 2 * 32 * SROW <= C::NBUF * C::STAGE, "staging blocks fit the tile memory");
+  half_t* const stg = smem + (size_t)wave * 2 * 32 * SROW;
 #pragma unroll
   for (int tt = 0; tt < NDT; ++tt)
 #pragma unroll
@@ -812,9 +816,22 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
         v1[e] = (half_t)(dq1[tt][4 * r4 + e] * p.sm_scale);
         v2[e] = (half_t)(dq2[tt][4 * r4 + e] * p.sm_scale);
       }
-      *reinterpret_cast<h4*>(o1 + 32 * tt + 8 * r4 + 4 * g) = v1;
-      *reinterpret_cast<h4*>(o2 + 32 * tt + 8 * r4 + 4 * g) = v2;
+      *reinterpret_cast<h4*>(stg + j * SROW + 32 * tt + 8 * r4 + 4 * g) = v1;
+      *reinterpret_cast<h4*>(stg + (32 + j) * SROW + 32 * tt + 8 * r4 + 4 * g) = v2;
     }
+  __builtin_amdgcn_wave_barrier();   // the rows are read back by other lanes of this wave only
+  constexpr int LPR = D / 8;         // lanes per row
+  constexpr int RPI = 64 / LPR;      // rows per instruction
+  half_t* const o1 = p.dq1 + (row0 + qt * BM + wave * 32) * D;
+  half_t* const o2 = p.dq2 + (row0 + qt * BM + wave * 32) * D;
+#pragma unroll
+  for (int k = 0; k < 32 / RPI; ++k) {
+    const int row = k * RPI + lane / LPR, ch = lane % LPR;
+    const u32x4 v1 = *reinterpret_cast<const u32x4*>(stg + row * SROW + 8 * ch);
+    const u32x4 v2 = *reinterpret_cast<const u32x4*>(stg + (32 + row) * SROW + 8 * ch);
+    *reinterpret_cast<u32x4*>(o1 + (size_t)row * D + 8 * ch) = v1;
+    *reinterpret_cast<u32x4*>(o2 + (size_t)row * D + 8 * ch) = v2;
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
