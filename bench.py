@@ -138,6 +138,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="capture the whole step in one HIP graph (torch.cuda.CUDAGraph) and time its replays: what a "
+                         "small problem costs once Python, the autograd engine and the allocator are out of the way")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -171,6 +174,31 @@ def main():
         y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"],
                                     causal=bool(cfg.get("causal")))
         y.backward(dy)
+
+    if args.graph:
+        # the whole step (forward, backward, gradient assignment) captured once and replayed: no Python,
+        # no autograd engine and no allocator in the timed region
+        eager_step = step
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                eager_step()
+        torch.cuda.current_stream().wait_stream(side)
+        for t in leaves:
+            t.grad = None
+        lam.grad = None
+        whole = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(whole):
+            if fwd_only:
+                with torch.no_grad():
+                    MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"])
+            else:
+                MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"],
+                                        causal=bool(cfg.get("causal"))).backward(dy)
+
+        def step():      # noqa: F811  (replaces the eager step)
+            whole.replay()
 
     for _ in range(args.warmup):
         step()
@@ -247,7 +275,7 @@ def main():
         "config": {"workload": "%s: diff-attn %s B%d H%d N%d D%d fp16 rms_norm=%s lambda=%.1f lambda_init=%.1f"
                                % (args.workload, "fwd" if fwd_only else "fwd+bwd", B, H, N, D, cfg["rms"], cfg["lam"],
                                   cfg["lambda_init"])
-                               + (" causal" if cfg.get("causal") else "")},
+                               + (" causal" if cfg.get("causal") else "") + (" (HIP graph replay)" if args.graph else "")},
         "frac_of_fp16_mfma_peak": value / PEAK_FP16_TFLOPS,
         # the K timed steps one by one (an event between steps): median and the 5 % / 95 % quantiles
         "ms_per_step_median": quantile(per_step, 0.5), "ms_per_step_p5": quantile(per_step, 0.05),
