@@ -244,9 +244,9 @@ def main():
         kernels_ms = {"fwd_kernel": event_time(launch_forward, k_iters, torch)}
         if not fwd_only:
             bwd_stage(15)()
+            # the fixed-order sum of the d(lambda) partials rides in the dK/dV launch of a full backward
             kernels_ms.update({
                 "bwd_prep_kernel": event_time(bwd_stage(1), k_iters, torch),
-                "bwd_dlambda_kernel": event_time(bwd_stage(2), k_iters, torch),
                 "bwd_dkdv_kernel": event_time(bwd_stage(4), k_iters, torch),
                 "bwd_dq_kernel": event_time(bwd_stage(8), k_iters, torch),
             })

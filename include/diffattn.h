@@ -154,6 +154,8 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
  * the backward with events on `stream`.  Stage bits, in execution order:
  *   DIFFATTN_STAGE_PREP    row preprocess: dX, row statistics, d(lambda) partials -> workspace
  *   DIFFATTN_STAGE_DLAMBDA fixed-order reduction of the partials -> dlambda
+ *                          (a launch of its own only when neither DKDV nor DQ is asked for: otherwise it
+ *                          rides in the first of their launches as one extra workgroup per lambda)
  *   DIFFATTN_STAGE_DKDV    dK1, dK2, dV   (reads the workspace written by PREP)
  *   DIFFATTN_STAGE_DQ      dQ1, dQ2       (reads the workspace written by PREP)
  * diffattn_backward(...) == diffattn_backward_stages(..., DIFFATTN_STAGE_ALL, stream).

@@ -9,7 +9,9 @@
 //                     dV += (P1 - lambda P2)^T dX, dK_t += s dS_t^T Q_t      (:410-424)
 //   bwd_dq_kernel     one workgroup per 128 queries, loops over all key tiles:
 //                     dQ_t += s dS_t K_t                                      (:426-436)
-//   bwd_dlambda_kernel  fixed-order sum of the partials into one fp16 value (one per head with per-head lambda)   (:573)
+//   d(lambda)         fixed-order sum of the partials into one fp16 value (one per head with per-head
+//                     lambda) (:573): one extra workgroup per value at the end of the first dK/dV or dQ
+//                     grid of the call, or bwd_dlambda_kernel when neither of them is launched
 //
 // The pre-norm row X is rebuilt as Y / ((1 - lambda_init) * rinv); only U2 = softmax(S2) V is
 // needed besides it, because U1 = X + lambda U2.
@@ -103,21 +105,23 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
   if (tid == 0) p.dlam_part[blockIdx.x] = red[0];
 }
 
-// Workgroup o of n_out sums the partials of the units o, o + n_out, o + 2 n_out, ...: with n_out = 1
+// Output o of n_out is the sum of the partials of the units o, o + n_out, o + 2 n_out, ...: with n_out = 1
 // every unit (one lambda), with n_out = H the units of head o (one lambda per head).  `per_unit`
-// consecutive partials belong to a unit.
-__global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restrict__ part, int per_unit, int n_units,
-                                                          half_t* out) {
-  __shared__ float red[256];
-  const int tid = threadIdx.x, o = blockIdx.x, n_out = gridDim.x;
+// consecutive partials belong to a unit.  One workgroup per output; its first 256 threads add in a fixed
+// order whatever the size of the workgroup, so the result does not depend on the kernel that hosts it.
+__device__ __forceinline__ void dlambda_reduce(const float* __restrict__ part, int per_unit, int n_units, half_t* out,
+                                               int o, int n_out, float* red) {
+  const int tid = threadIdx.x;
   const int n = (n_units / n_out) * per_unit;        // partials this workgroup sums
   float acc = 0.f;
-  if (n_out == 1) {
-    for (int i = tid; i < n; i += 256) acc += part[i];
-  } else {
-    for (int i = tid; i < n; i += 256) acc += part[(size_t)(o + (i / per_unit) * n_out) * per_unit + i % per_unit];
+  if (tid < 256) {
+    if (n_out == 1) {
+      for (int i = tid; i < n; i += 256) acc += part[i];
+    } else {
+      for (int i = tid; i < n; i += 256) acc += part[(size_t)(o + (i / per_unit) * n_out) * per_unit + i % per_unit];
+    }
+    red[tid] = acc;
   }
-  red[tid] = acc;
   __syncthreads();
 #pragma unroll
   for (int s = 128; s >= 1; s >>= 1) {
@@ -126,6 +130,21 @@ __global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restric
   }
   if (tid == 0) out[o] = (half_t)red[0];
 }
+
+__global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restrict__ part, int per_unit, int n_units,
+                                                          half_t* out) {
+  __shared__ float red[256];
+  dlambda_reduce(part, per_unit, n_units, out, blockIdx.x, gridDim.x, red);
+}
+
+// The dK/dV and dQ kernels can host that reduction in p.dlam_fold extra workgroups at the end of their grid
+// (one launch less per backward): such a workgroup does nothing else.
+#define DA_HOST_DLAMBDA(smem_)                                                                                  \
+  if (p.dlam_fold && (int)blockIdx.x >= (int)gridDim.x - p.dlam_fold) {                                         \
+    dlambda_reduce(p.dlam_part, p.n_part / p.BH, p.BH, p.dlambda, (int)blockIdx.x - ((int)gridDim.x - p.dlam_fold), \
+                   p.dlam_fold, reinterpret_cast<float*>(smem_));                                               \
+    return;                                                                                                     \
+  }
 
 // ------------------------------------------------------------------------------------------------
 template <int D>
@@ -162,6 +181,8 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   constexpr bool DO_V = (MODE != 2), DO_K = (MODE != 1);
 
   __shared__ __attribute__((aligned(16))) half_t smem[C::NBUF * C::STAGE];
+  static_assert(sizeof(smem) >= 256 * sizeof(float), "the hosted reduction uses the tile memory");
+  DA_HOST_DLAMBDA(smem)
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -173,7 +194,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     const UnitBlock ub = longest_first(blockIdx.x, p.BH);
     bh = ub.unit; kt = ub.rank;
   } else {
-    const int tile = xcd_remap(blockIdx.x, gridDim.x);
+    const int tile = xcd_remap(blockIdx.x, gridDim.x - p.dlam_fold);
     bh = tile / n_kt; kt = tile % n_kt;
   }
   const size_t rows = (size_t)p.BH * p.N;
@@ -619,6 +640,8 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
 
   __shared__ __attribute__((aligned(16))) half_t smem[C::NBUF * C::STAGE];
+  static_assert(sizeof(smem) >= 256 * sizeof(float), "the hosted reduction uses the tile memory");
+  DA_HOST_DLAMBDA(smem)
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -630,7 +653,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
     const UnitBlock ub = longest_first(blockIdx.x, p.BH);
     bh = ub.unit; qt = n_qt - 1 - ub.rank;
   } else {
-    const int tile = xcd_remap(blockIdx.x, gridDim.x);
+    const int tile = xcd_remap(blockIdx.x, gridDim.x - p.dlam_fold);
     bh = tile / n_qt; qt = tile % n_qt;
   }
   const size_t rows = (size_t)p.BH * p.N;
@@ -872,9 +895,14 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
 
 // ------------------------------------------------------------------------------------------------
 template <int D>
-static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
+static hipError_t launch_bwd_t(const BwdParams& p_in, hipStream_t stream) {
+  BwdParams p = p_in;
   const int n_prep = bwd_num_partials(p.BH, p.N, D);
   hipError_t e = hipSuccess;
+  // the d(lambda) reduce rides in the first dK/dV or dQ launch when there is one, else it is a launch of its own
+  const int n_lambda = p.lambda_stride ? p.H : 1;
+  bool fold = (p.stages & 2u) && (p.stages & 12u);
+  p.dlam_fold = 0;
   if (p.stages & 1u) {
     if (p.rms_norm)
       hipLaunchKernelGGL((bwd_prep_kernel<D, true>), dim3(n_prep), dim3(256), 0, stream, p);
@@ -882,15 +910,18 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
       hipLaunchKernelGGL((bwd_prep_kernel<D, false>), dim3(n_prep), dim3(256), 0, stream, p);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
-  if (p.stages & 2u) {
-    hipLaunchKernelGGL(bwd_dlambda_kernel, dim3(p.lambda_stride ? p.H : 1), dim3(256), 0, stream,
+  if ((p.stages & 2u) && !fold) {
+    hipLaunchKernelGGL(bwd_dlambda_kernel, dim3(n_lambda), dim3(256), 0, stream,
                        p.dlam_part, n_prep / p.BH, p.BH, p.dlambda);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 4u) {
-    const dim3 grid(p.BH * (p.N / DkvCfg<D>::BK)), block(DkvCfg<D>::NT);
+    const dim3 block(DkvCfg<D>::NT);
     auto launch_mode = [&](auto mode_tag) {
       constexpr int M = decltype(mode_tag)::value;
+      p.dlam_fold = fold ? n_lambda : 0;
+      fold = false;
+      const dim3 grid(p.BH * (p.N / DkvCfg<D>::BK) + p.dlam_fold);
       if (p.drop.threshold) {
         if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, true, true>), grid, block, 0, stream, p);
         else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, false, true>), grid, block, 0, stream, p);
@@ -917,6 +948,9 @@ static hipError_t launch_bwd_t(const BwdParams& p, hipStream_t stream) {
     bool wide = false;
     auto launch_dq = [&](auto nw_tag, dim3 grid, dim3 block) {
       constexpr int NWV = decltype(nw_tag)::value;
+      p.dlam_fold = fold ? n_lambda : 0;
+      fold = false;
+      grid.x += p.dlam_fold;
       if (p.drop.threshold) {
         if (p.causal)            hipLaunchKernelGGL((bwd_dq_kernel<D, NWV, 1, true>), grid, block, 0, stream, p);
         else if (p.n_keys < p.N) hipLaunchKernelGGL((bwd_dq_kernel<D, NWV, 2, true>), grid, block, 0, stream, p);

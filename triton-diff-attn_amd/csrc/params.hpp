@@ -48,6 +48,7 @@ struct BwdParamsT {
   int causal;
   int n_keys;                   // keys n_keys..N-1 are padding (N when there is none)
   unsigned stages;              // bit 0 row preprocess, 1 d(lambda) reduce, 2 dK/dV, 3 dQ
+  int dlam_fold;                // set by the launcher: extra workgroups at the end of a dK/dV or dQ grid that do the d(lambda) reduce
   int H;                        // heads per batch entry: unit bh belongs to head bh % H
   int lambda_stride;            // 0: one lambda; 1: one per head
   Strides sqk, sv, sy, sdy;     // layouts of q1,q2,k1,k2 / v / y / dy; everything else is dense
