@@ -48,3 +48,16 @@ def test_constant_inputs_and_zero_gradient():
     q1, q2, k1, k2, v, dy = make_inputs(B, H, N, D, seed=45)
     y, grads = run_kernel(q1, q2, k1, k2, v, 0.5, 0.8, True, torch.zeros_like(dy))
     assert all(g.abs().max().item() == 0 for g in grads)     # zero upstream gradient gives exactly zero gradients
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_upstream_gradient_with_a_loss_scale(D):
+    """dy multiplied by 1024, as a gradient scaler does: dP - delta reaches 1e5, beyond the 16-bit range, while
+    dS = P (dP - delta) and the gradients (about 2000) stay well inside it.  Gradients are linear in dy."""
+    q1, q2, k1, k2, v, dy = make_inputs(1, 2, 1024, D, seed=46)
+    scale = 1024.0
+    y, grads = run_kernel(q1, q2, k1, k2, v, 0.5, 0.8, True, (dy * scale).half())
+    ref = orc.forward_backward(q1, q2, k1, k2, v, torch.tensor([0.5], dtype=torch.float16), dy, 0.8, True)
+    for name, g, r in zip(("dq1", "dq2", "dk1", "dk2", "dv"), grads, ref[1:6]):
+        assert torch.isfinite(g).all(), name
+        assert rel_to_max(g.float() / scale, r) <= GRAD_RTOL, name

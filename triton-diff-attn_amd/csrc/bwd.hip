@@ -369,9 +369,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
       }
       return;
     }
-    if constexpr ((MODE == 0) && !DROP) {
-      asm volatile("" : "+v"(t.p1[r]), "+v"(t.p2[r]));                 // computed here, not moved to their use
-    } else if constexpr (DO_K) {
+    if constexpr (DO_K) {
       t.u[r] = __builtin_fmaf(-lam, in.dp[r], st3[r % 4]);
       asm volatile("" : "+v"(t.p1[r]), "+v"(t.p2[r]), "+v"(t.u[r]));   // computed here, not moved to its use
     } else {
@@ -403,31 +401,12 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
       out.d2[r / 8][r % 8 - 1] = (half_t)t.ds2[r - 1]; out.d2[r / 8][r % 8] = (half_t)t.ds2[r];
     }
   };
-  // Packed form of stages 2 and 3 for the one-pass kernel without dropout: rows r-1 and r (r odd) as
-  // pairs of 16-bit values -- 4 conversions and 4 packed operations instead of 8 fp32 operations and
-  // 3 conversions; dS and P are rounded to 16 bits for their products anyway.
-  constexpr bool PACKED_EW = (MODE == 0) && !DROP;
-  const h2 neg_lam2 = {(half_t)(-lam), (half_t)(-lam)};
-  auto ew23 = [&](int r, const f4v& st3, const Scores& in, const RowTmp& t, Packed& out) {
-    const h2 P1 = {(half_t)t.p1[r - 1], (half_t)t.p1[r]}, P2 = {(half_t)t.p2[r - 1], (half_t)t.p2[r]};
-    const h2 DP = {(half_t)in.dp[r - 1], (half_t)in.dp[r]};                 // dP - delta1 (accumulator init)
-    const h2 ST = {(half_t)st3[(r - 1) % 4], (half_t)st3[r % 4]};
-    const h2 U = neg_lam2 * DP + ST;                                         // -lambda dP - delta2
-    const h2 D1 = P1 * DP, D2 = P2 * U, PC = neg_lam2 * P2 + P1;
-    out.d1[r / 8][r % 8 - 1] = D1[0]; out.d1[r / 8][r % 8] = D1[1];
-    out.d2[r / 8][r % 8 - 1] = D2[0]; out.d2[r / 8][r % 8] = D2[1];
-    out.pc[r / 8][r % 8 - 1] = PC[0]; out.pc[r / 8][r % 8] = PC[1];
-  };
   // slot s of the skewed schedule: stage 1 of row s, stage 2 of row s-1, stage 3 of the pair ending at row s-2
   auto ew_slot = [&](int s, const f4v (&st)[4], const f4v (&st2)[4], const Scores& in, RowTmp& t, Packed& out, auto masked_tag,
                      int rel, int qbase) {
     if (s < 16) ew1(s, st[s / 4], st2[s / 4], in, t, masked_tag, rel, qbase);
-    if constexpr (PACKED_EW) {
-      if (s >= 2 && s - 2 < 16 && ((s - 2) & 1)) ew23(s - 2, st[(s - 2) / 4], in, t, out);
-    } else {
-      if (s >= 1 && s - 1 < 16) ew2(s - 1, in, t);
-      if (s >= 2 && s - 2 < 16 && ((s - 2) & 1)) ew3(s - 2, t, out);
-    }
+    if (s >= 1 && s - 1 < 16) ew2(s - 1, in, t);
+    if (s >= 2 && s - 2 < 16 && ((s - 2) & 1)) ew3(s - 2, t, out);
   };
   // B fragment (transposing read) of accumulate product m of sub-tile qs: m = kk*NACC1 + slot, where
   // the slots of a 16-query k-step are the dV feature tiles followed by the dK1/dK2 feature tiles
@@ -799,8 +778,6 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       __builtin_amdgcn_sched_barrier(0);
       h8 b1[2], b2[2];
       unsigned w1 = 0, w2 = 0;
-      float p1_prev = 0.f, p2_prev = 0.f;
-      const h2 NEGLAM2 = {(half_t)(-lam), (half_t)(-lam)}, DE2 = {(half_t)de2, (half_t)de2};
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float p1 = fast_exp2(s1[r] + nl1);
@@ -820,22 +797,11 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
           b1[r / 8][r % 8] = (half_t)(p1 * (d1 + de1));                                             // c m1 dP - delta1
           b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, d2, __builtin_fmaf(-lam, de1, de2)));   // -lambda c m2 dP - delta2
         } else {
-          if constexpr (D <= 64) {
-            // pairs of rows in packed 16-bit arithmetic (half the VALU instructions): dS is rounded
-            // to 16 bits for its product anyway.  D = 128 has no registers to spare for the pairing.
-            if (r & 1) {
-              const h2 P1 = {(half_t)p1_prev, (half_t)p1}, P2 = {(half_t)p2_prev, (half_t)p2};
-              const h2 DPC = {(half_t)(dp[r - 1] + de1), (half_t)(dp[r] + de1)};      // statistic 2 is -delta1
-              const h2 U = NEGLAM2 * DPC + DE2;                                       // statistic 3 is -(lambda*delta1 + delta2)
-              const h2 B1 = P1 * DPC, B2 = P2 * U;
-              b1[r / 8][r % 8 - 1] = B1[0]; b1[r / 8][r % 8] = B1[1];
-              b2[r / 8][r % 8 - 1] = B2[0]; b2[r / 8][r % 8] = B2[1];
-            } else { p1_prev = p1; p2_prev = p2; }
-          } else {
-            const float dpc = dp[r] + de1;                  // statistic 2 is -delta1
-            b1[r / 8][r % 8] = (half_t)(p1 * dpc);
-            b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dpc, de2));   // statistic 3 is -(lambda*delta1 + delta2)
-          }
+          // in fp32 up to the rounding of dS itself: dP - delta alone may exceed the 16-bit range when the
+          // upstream gradient carries a loss scale, while its product with the probability does not
+          const float dpc = dp[r] + de1;                  // statistic 2 is -delta1
+          b1[r / 8][r % 8] = (half_t)(p1 * dpc);
+          b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dpc, de2));   // statistic 3 is -(lambda*delta1 + delta2)
         }
       }
 #pragma unroll
