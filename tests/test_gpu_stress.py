@@ -50,12 +50,13 @@ def test_constant_inputs_and_zero_gradient():
     assert all(g.abs().max().item() == 0 for g in grads)     # zero upstream gradient gives exactly zero gradients
 
 
+@pytest.mark.parametrize("scale", [1024.0, 1e-3])
 @pytest.mark.parametrize("D", [32, 64, 128])
-def test_upstream_gradient_with_a_loss_scale(D):
+def test_upstream_gradient_with_a_loss_scale(D, scale):
     """dy multiplied by 1024, as a gradient scaler does: dP - delta reaches 1e5, beyond the 16-bit range, while
-    dS = P (dP - delta) and the gradients (about 2000) stay well inside it.  Gradients are linear in dy."""
+    dS = P (dP - delta) and the gradients (about 2000) stay well inside it.  Gradients are linear in dy.
+    And the other end: an upstream gradient of order 1e-3, whose dS values are fp16 subnormals."""
     q1, q2, k1, k2, v, dy = make_inputs(1, 2, 1024, D, seed=46)
-    scale = 1024.0
     y, grads = run_kernel(q1, q2, k1, k2, v, 0.5, 0.8, True, (dy * scale).half())
     ref = orc.forward_backward(q1, q2, k1, k2, v, torch.tensor([0.5], dtype=torch.float16), dy, 0.8, True)
     for name, g, r in zip(("dq1", "dq2", "dk1", "dk2", "dv"), grads, ref[1:6]):
