@@ -158,9 +158,17 @@ struct DkvCfg {
   static constexpr int X_TILE = BQ * DV;
   static constexpr int STAT = 4 * BQ * 2;      // 4 float arrays, counted in halfs
   static constexpr int STAGE = 2 * Q_TILE + X_TILE + STAT;
-  // a staged tile is read until half a step after its last sub-tile was scored while the tile two
-  // ahead is already being fetched: three buffers, four when a tile is a single sub-tile
-  static constexpr int NBUF = (BQ == 32) ? 4 : 3;
+  // LDS map in bytes: the ring buffers of each kind of tile are contiguous, so that any buffer of a kind
+  // is within the 64 KiB reach of an LDS instruction's immediate offset from one per-lane address
+  static constexpr int QBUF = 2 * Q_TILE * 2, XBUF = X_TILE * 2, SBUF = STAT * 2;   // one ring buffer of Q1|Q2, dX, statistics
+  // A staged tile is read until half a step after its last sub-tile was scored while the tile after
+  // the next is already being fetched, which takes three buffers; there are four so that the ring
+  // position of every step is known at compile time (the loop is unrolled over one turn of the ring,
+  // and the number of steps is a multiple of four): every LDS address is then a per-lane register
+  // plus an immediate offset, with no address arithmetic inside the loop.
+  static constexpr int NBUF = 4;
+  static constexpr int XBASE = NBUF * QBUF, SBASE = XBASE + NBUF * XBUF;
+  static_assert(NBUF * QBUF <= 65536 && NBUF * XBUF <= 65536, "immediate offsets reach every buffer");
 };
 
 // dK_t and dV for one block of keys.  Products are formed as [queries x keys] so that a lane owns
@@ -257,21 +265,54 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   constexpr int XH = (XTile::PER + 1) / 2;
 
   auto stage = [&](int qt, int buf, int part) {
-    half_t* b = smem + buf * C::STAGE;
+    half_t* bq = smem + buf * (C::QBUF / 2);
+    half_t* bx = smem + (C::XBASE + buf * C::XBUF) / 2;
     if (part == 0) {
-      QTile::issue_at(gq1 + (size_t)qt * BQ * qk_n, b, wave, lane, q_off, qk_n);
-      if (wave == 0 && lane < BQ) async_copy16(reinterpret_cast<const half_t*>(gstat + (size_t)qt * BQ), stat_off, b + 2 * C::Q_TILE + C::X_TILE);
+      QTile::issue_at(gq1 + (size_t)qt * BQ * qk_n, bq, wave, lane, q_off, qk_n);
+      if (wave == 0 && lane < BQ) async_copy16(reinterpret_cast<const half_t*>(gstat + (size_t)qt * BQ), stat_off, smem + (C::SBASE + buf * C::SBUF) / 2);
     } else if (part == 1) {
-      QTile::issue_at(gq2 + (size_t)qt * BQ * qk_n, b + C::Q_TILE, wave, lane, q_off, qk_n);
+      QTile::issue_at(gq2 + (size_t)qt * BQ * qk_n, bq + C::Q_TILE, wave, lane, q_off, qk_n);
     } else if (part == 2) {
-      XTile::template issue<0, XH>(gx + (size_t)qt * BQ * DV, b + 2 * C::Q_TILE, wave, lane);
+      XTile::template issue<0, XH>(gx + (size_t)qt * BQ * DV, bx, wave, lane);
     } else {
-      XTile::template issue<XH, XTile::PER>(gx + (size_t)qt * BQ * DV, b + 2 * C::Q_TILE, wave, lane);
+      XTile::template issue<XH, XTile::PER>(gx + (size_t)qt * BQ * DV, bx, wave, lane);
     }
   };
 
   const int tr_row = 4 * g + ((lane & 15) >> 2);  // transposing reads: row inside a 16-row k-step
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  // Per-lane LDS byte addresses, computed once.  The XOR swizzle makes the address of a fragment a
+  // different function of the lane for every 16-byte chunk column, so there is one register per chunk
+  // column a lane ever reads; everything else (ring buffer, Q1 or Q2, sub-tile, k-step of 16 rows) is a
+  // multiple of 16 rows, which the swizzle does not see, and travels in the instruction's immediate offset.
+  const unsigned lds0 = (unsigned)(unsigned long)((DA_LDS char*)smem);
+  unsigned qb[NKS], xb[NKV], qtr[NDT][2], xtr[NVT][2], stb;
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) qb[ks] = lds0 + 2u * (unsigned)swz_off<D>(j, 16 * ks + 8 * g);
+#pragma unroll
+  for (int kv = 0; kv < NKV; ++kv) xb[kv] = lds0 + C::XBASE + 2u * (unsigned)swz_off<DV>(j, 16 * kv + 8 * g);
+#pragma unroll
+  for (int tt = 0; tt < NDT; ++tt)
+#pragma unroll
+    for (int e = 0; e < 2; ++e) qtr[tt][e] = lds0 + 2u * (unsigned)swz_off<D>(tr_row + 8 * e, 32 * tt + tr_col);
+#pragma unroll
+  for (int tt = 0; tt < NVT; ++tt)
+#pragma unroll
+    for (int e = 0; e < 2; ++e) xtr[tt][e] = lds0 + C::XBASE + 2u * (unsigned)swz_off<DV>(tr_row + 8 * e, 32 * tt + tr_col);
+  stb = lds0 + C::SBASE + 16u * (unsigned)g;
+  // kept as they are: the compiler neither folds constants into them nor recomputes them in the loop
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) asm volatile("" : "+v"(qb[ks]));
+#pragma unroll
+  for (int kv = 0; kv < NKV; ++kv) asm volatile("" : "+v"(xb[kv]));
+#pragma unroll
+  for (int tt = 0; tt < NDT; ++tt) asm volatile("" : "+v"(qtr[tt][0]), "+v"(qtr[tt][1]));
+#pragma unroll
+  for (int tt = 0; tt < NVT; ++tt) asm volatile("" : "+v"(xtr[tt][0]), "+v"(xtr[tt][1]));
+  asm volatile("" : "+v"(stb));
+  auto lds_h8 = [](unsigned addr, int off) -> h8 { return lds_read_at<h8>(addr, off); };
+  auto lds_tr = [](unsigned addr, int off) -> h4 { return lds_read_tr_at(addr, off); };
 
   // The loop runs over 32-query sub-tiles i (SPT per staged tile), software-pipelined inside the
   // wave.  Step i interleaves, instruction group by instruction group,
@@ -292,13 +333,11 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   // the three accumulation chains advance together; without dP (MODE 1) S1 and S2 alternate.
   static_assert(NKV == 2 * NKS, "every second product belongs to dP");
   auto prod_frag = [&](int buf, int qs, int k) -> h8 {
-    const half_t* sQ1 = smem + buf * C::STAGE;
     if (!DO_K || (k & 1)) {
       const int t = DO_K ? (k >> 1) : k;
-      const half_t* sQ = sQ1 + (t & 1) * C::Q_TILE;
-      return *reinterpret_cast<const h8*>(sQ + swz_off<D>(qs * 32 + j, 16 * (t >> 1) + 8 * g));
+      return lds_h8(qb[t >> 1], buf * C::QBUF + (t & 1) * C::Q_TILE * 2 + qs * 32 * D * 2);
     }
-    return *reinterpret_cast<const h8*>(sQ1 + 2 * C::Q_TILE + swz_off<DV>(qs * 32 + j, 16 * (k >> 1) + 8 * g));
+    return lds_h8(xb[k >> 1], buf * C::XBUF + qs * 32 * DV * 2);
   };
   // The dropout instantiations spill a few registers; there the products are issued as ordinary
   // (compiler-visible) matrix instructions, so that the compiler places every wait state itself:
@@ -316,8 +355,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   // 3: -(lambda*delta1 + delta2).  Statistics 0..2 are the initial accumulator values of the three
   // product chains, so the matrix unit delivers s1 - lse1, s2 - lse2 (log2 units) and dP - delta1.
   auto stat4 = [&](int buf, int qs, int which, int r4) -> f4v {
-    const float* sStat = reinterpret_cast<const float*>(smem + buf * C::STAGE + 2 * C::Q_TILE + C::X_TILE);
-    return *reinterpret_cast<const f4v*>(sStat + which * BQ + qs * 32 + 8 * r4 + 4 * g);
+    return lds_read_at<f4v>(stb, buf * C::SBUF + (which * BQ + qs * 32 + 8 * r4) * 4);
   };
   auto results_ready = [&](Scores& s) {
     if constexpr (DO_K) mfma_results_ready(s.s1, s.s2, s.dp);
@@ -416,18 +454,15 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   static_assert(NPROD % NACC == 0, "a whole number of score products per accumulate product");
   constexpr int RATIO = NPROD / NACC;
   auto acc_frag = [&](int buf, int qs, int m) -> h8 {
-    const half_t* sQ1 = smem + buf * C::STAGE;
     const int kk = m / NACC1, slot = m % NACC1;
-    const int rbase = qs * 32 + 16 * kk + tr_row;
+    const int row0 = qs * 32 + 16 * kk;
     if (slot < NSV) {
-      const half_t* sX = sQ1 + 2 * C::Q_TILE;
-      return join(lds_read_tr(sX + swz_off<DV>(rbase, 32 * slot + tr_col)),
-                  lds_read_tr(sX + swz_off<DV>(rbase + 8, 32 * slot + tr_col)));
+      const int off = buf * C::XBUF + row0 * DV * 2;
+      return join(lds_tr(xtr[slot][0], off), lds_tr(xtr[slot][1], off));
     }
     const int t2 = slot - NSV;
-    const half_t* sQ = sQ1 + (t2 & 1) * C::Q_TILE;
-    return join(lds_read_tr(sQ + swz_off<D>(rbase, 32 * (t2 >> 1) + tr_col)),
-                lds_read_tr(sQ + swz_off<D>(rbase + 8, 32 * (t2 >> 1) + tr_col)));
+    const int off = buf * C::QBUF + (t2 & 1) * C::Q_TILE * 2 + row0 * D * 2;
+    return join(lds_tr(qtr[t2 >> 1][0], off), lds_tr(qtr[t2 >> 1][1], off));
   };
   auto acc_mfma = [&](int m, h8 bfrag, const Packed& in) {
     const int kk = m / NACC1, slot = m % NACC1;
@@ -439,10 +474,13 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
 
   const int n_qt = p.N / BQ;
   const int n_sub = p.N / 32;
-  auto buf_of = [](int tile) { return tile % C::NBUF; };
   // first sub-tile and tile of the loop: with the causal mask no query before the key block matters
   const int i0 = CAUSAL ? kt * (BK / 32) : 0;
   const int t0 = i0 / SPT;
+  // Tile t0 + k lives in buffer k % NBUF.  Step number s of the loop (sub-tile i0 + s) is at ring
+  // position s % RING; the positions of its three sub-tiles follow from that at compile time.
+  constexpr int NBUF = C::NBUF, RING = SPT * NBUF, HALF = RING / 2;
+  static_assert(HALF % 2 == 0 && 4 % HALF == 0, "half a turn is an even number of steps and divides the step count");
 
   // One step.  Chunk k holds score product k of sub-tile (bufn, qsn), every RATIO-th chunk also
   // accumulate product (k/RATIO + NACC/2) % NACC -- the upper query half of sub-tile (bufp, qsp)
@@ -453,7 +491,9 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   static_assert(NPROD % 16 == 0 || 16 % NPROD == 0, "rows are spread evenly over the products");
   constexpr int AHEAD = DROP ? 1 : 3;          // B fragments requested ahead of their product
   auto fused = [&](int bufn, int qsn, Scores& s_nxt, int bufc, int qsc, const Scores& s_cur, Packed& pk,
-                   int bufp, int qsp, int tile_next, int buf_next, bool fetch, auto masked_tag, int rel, int qbase) {
+                   int bufp, int qsp, int tile_next, auto buf_next_tag, auto fetch_tag, auto masked_tag, int rel, int qbase) {
+    constexpr int buf_next = decltype(buf_next_tag)::value;
+    constexpr bool fetch = decltype(fetch_tag)::value;
     constexpr int NSLOT = 18;                  // 16 rows + 2 slots of pipeline drain
     constexpr int LEAD = 2;                    // slots run before the first product
     // rows 0..7 are packed by slot 9, which must precede the first product that reads them
@@ -499,36 +539,44 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     results_ready(s_nxt);
   };
 
-  // step i: compile-time positions of sub-tiles i+1, i, i-1 inside their tiles
-  auto step = [&](int i, auto subn_tag, const Scores& s_cur, Scores& s_nxt, Packed& pk, auto masked_tag) {
-    constexpr int SUBN = decltype(subn_tag)::value;           // (i + 1) % SPT
-    constexpr int SUBC = (SUBN + SPT - 1) % SPT;              // i % SPT
-    constexpr int SUBP = (SUBN + 2 * SPT - 2) % SPT;          // (i - 1) % SPT
-    const bool more = (i + 1 < n_sub);
-    const int tn = (more ? i + 1 : i) / SPT, tc = i / SPT, tp = (i > i0 ? i - 1 : i0) / SPT;
-    const bool opens = (SUBN == 0 && more);
-    if (opens) {
+  // step i at ring position POS: sub-tile i+1 is scored, sub-tile i gets its element-wise work, and the
+  // accumulate products run over the upper half of sub-tile i-1 and the lower half of sub-tile i
+  auto step = [&](int i, auto pos_tag, const Scores& s_cur, Scores& s_nxt, Packed& pk, auto masked_tag) {
+    constexpr int POS = decltype(pos_tag)::value;
+    constexpr int SUBN = (POS + 1) % SPT, SUBC = POS % SPT, SUBP = (POS + RING - 1) % SPT;
+    constexpr int BUFN = ((POS + 1) / SPT) % NBUF, BUFC = POS / SPT, BUFP = ((POS + RING - 1) / SPT) % NBUF;
+    constexpr bool opens = (SUBN == 0);
+    const int tn = (i + 1) / SPT;
+    if constexpr (opens) {
       // sub-tile i+1 opens tile tn: its data must have landed; tile tn+1 is fetched during this step
       wait_async_tiles();
       __syncthreads();
     }
-    const int tl = (tn + 1 < n_qt) ? tn + 1 : tn;             // past the end: harmless re-read
-    // past the end the last sub-tile is scored again and the result is never used; before the
-    // start the all-zero upper operand half is accumulated against the first tile
-    fused(buf_of(tn), more ? SUBN : SUBC, s_nxt, buf_of(tc), SUBC, s_cur, pk,
-          buf_of(tp), (i > i0) ? SUBP : 0, tl, buf_of(tn + 1), opens, masked_tag, key - 32 * i - 4 * g, 32 * i + 4 * g);
+    // Past the end the last tile is fetched and scored again and the result is never used.  In front of
+    // the first sub-tile the all-zero upper operand half is accumulated against the zero-filled last buffer.
+    const int tl = (tn + 1 < n_qt) ? tn + 1 : n_qt - 1;
+    fused(BUFN, SUBN, s_nxt, BUFC, SUBC, s_cur, pk, BUFP, SUBP, tl, std::integral_constant<int, (BUFN + 1) % NBUF>{},
+          std::integral_constant<bool, opens>{}, masked_tag, key - 32 * i - 4 * g, 32 * i + 4 * g);
   };
 
-  // prologue: the first tile, then start fetching the second; scores of the first sub-tile
+  // prologue: the last buffer, which the first step reads as "the sub-tile before the first", is cleared
+  // (uninitialised LDS could hold NaN patterns, and 0 * NaN would poison the sums); the first tile is
+  // fetched, then the second starts; scores of the first sub-tile
+  const bool head_half = (HALF == 4) && (((n_sub - i0) / HALF) & 1);   // with HALF == 2 the steps are whole turns
+  const int b0 = head_half ? NBUF / 2 : 0;          // buffer of the first tile
   {
-    const int b0 = buf_of(t0);
-    stage(t0, b0, 0); stage(t0, b0, 1); stage(t0, b0, 2); stage(t0, b0, 3);
+    const int bz = (b0 + NBUF - 1) % NBUF;          // the buffer in front of the first tile's
+    u32x4* zq = reinterpret_cast<u32x4*>(smem + bz * (C::QBUF / 2));
+    u32x4* zx = reinterpret_cast<u32x4*>(smem + (C::XBASE + bz * C::XBUF) / 2);
+    for (int k = tid; k < C::QBUF / 16; k += C::NT) zq[k] = u32x4{0u, 0u, 0u, 0u};
+    for (int k = tid; k < C::XBUF / 16; k += C::NT) zx[k] = u32x4{0u, 0u, 0u, 0u};
   }
+  stage(t0, b0, 0); stage(t0, b0, 1); stage(t0, b0, 2); stage(t0, b0, 3);
   wait_async_tiles();
   __syncthreads();
   {
-    const int t1 = (t0 + 1 < n_qt) ? t0 + 1 : t0, b1 = buf_of(t0 + 1);
-    stage(t1, b1, 0); stage(t1, b1, 1); stage(t1, b1, 2); stage(t1, b1, 3);
+    const int t1 = (t0 + 1 < n_qt) ? t0 + 1 : t0;
+    stage(t1, b0 + 1, 0); stage(t1, b0 + 1, 1); stage(t1, b0 + 1, 2); stage(t1, b0 + 1, 3);
   }
   Scores sa, sb;
   Packed pk;
@@ -536,31 +584,56 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
     for (int e = 0; e < 8; ++e) { pk.pc[kk][e] = (half_t)0.f; pk.d1[kk][e] = (half_t)0.f; pk.d2[kk][e] = (half_t)0.f; }
-  init_scores(buf_of(t0), 0, sa);
+  if (head_half) {
+    init_scores(NBUF / 2, 0, sa);
 #pragma unroll
-  for (int k = 0; k < NPROD; ++k) prod_mfma(k, prod_frag(buf_of(t0), 0, k), sa);
+    for (int k = 0; k < NPROD; ++k) prod_mfma(k, prod_frag(NBUF / 2, 0, k), sa);
+  } else {
+    init_scores(0, 0, sa);
+#pragma unroll
+    for (int k = 0; k < NPROD; ++k) prod_mfma(k, prod_frag(0, 0, k), sa);
+  }
   results_ready(sa);
 
-  constexpr std::integral_constant<int, 1 % SPT> even_tag{};   // position of sub-tile i+1 in its tile, i even
-  constexpr std::integral_constant<int, 2 % SPT> odd_tag{};
+  // two steps, starting at the even ring position P0 with the scores of sub-tile i in sa
+  auto two_steps = [&](int i, auto p0_tag, auto masked_tag) {
+    constexpr int P0 = decltype(p0_tag)::value;
+    step(i, std::integral_constant<int, P0>{}, sa, sb, pk, masked_tag);
+    step(i + 1, std::integral_constant<int, P0 + 1>{}, sb, sa, pk, masked_tag);
+  };
+  auto half_turn = [&](int i, auto h0_tag, auto masked_tag) {
+    constexpr int H0 = decltype(h0_tag)::value;
+    two_steps(i, std::integral_constant<int, H0>{}, masked_tag);
+    if constexpr (HALF == 4) two_steps(i + 2, std::integral_constant<int, H0 + 2>{}, masked_tag);
+  };
+  // The steps, a multiple of four, are an odd or even number of half turns; the loop below runs whole
+  // turns, so an odd half turn comes first, at the ring's second half (the prologue has put the first
+  // tile into the buffer that goes with it).  With the causal mask the key block's own four sub-tiles
+  // come first and straddle the diagonal: wave w masks sub-tiles i0 .. i0+w.
+  static_assert(!CAUSAL || BK == 128, "four diagonal sub-tiles per key block");
+  constexpr std::integral_constant<int, 0> first_half{};
+  constexpr std::integral_constant<int, HALF> second_half{};
+  constexpr std::integral_constant<bool, CAUSAL> head_masked{};
   int i = i0;
-  if constexpr (CAUSAL) {
-    // the key block's own four sub-tiles straddle the diagonal: wave w masks sub-tiles i0 .. i0+w
-    static_assert(BK == 128, "four diagonal sub-tiles per key block");
-    step(i0, even_tag, sa, sb, pk, std::true_type{});
-    step(i0 + 1, odd_tag, sb, sa, pk, std::true_type{});
-    step(i0 + 2, even_tag, sa, sb, pk, std::true_type{});
-    step(i0 + 3, odd_tag, sb, sa, pk, std::true_type{});
-    i = i0 + 4;
+  if (head_half) {
+    half_turn(i, second_half, head_masked);
+    i += HALF;
+  } else if constexpr (CAUSAL) {
+    half_turn(i, first_half, std::true_type{});
+    half_turn(i + HALF, second_half, std::integral_constant<bool, HALF == 2>{});
+    i += RING;
   }
-  for (; i < n_sub; i += 2) {   // an even number of sub-tiles remains
-    step(i, even_tag, sa, sb, pk, std::false_type{});
-    step(i + 1, odd_tag, sb, sa, pk, std::false_type{});
+#pragma nounroll
+  while (i < n_sub) {
+    half_turn(i, first_half, std::false_type{});
+    half_turn(i + HALF, second_half, std::false_type{});
+    i += RING;
   }
-  // upper query half of the last sub-tile
+  // upper query half of the last sub-tile, at the last ring position
 #pragma unroll
-  for (int m = NACC / 2; m < NACC; ++m) acc_mfma(m, acc_frag(buf_of((n_sub - 1) / SPT), (n_sub - 1) % SPT, m), pk);
+  for (int m = NACC / 2; m < NACC; ++m) acc_mfma(m, acc_frag((RING - 1) / SPT, (RING - 1) % SPT, m), pk);
 
+  wait_async_tiles();   // the re-fetch issued by the last step has nothing left to land in after the kernel
   // accumulator tile tt: column = 32*tt + j (feature), register r = key row 8*(r/4) + 4g + (r%4)
   const size_t krow0 = row0 + (size_t)kt * BK + wave * 32;
   if constexpr (DO_V) {

@@ -127,6 +127,23 @@ __device__ __forceinline__ h4 lds_read_tr(const half_t* p) {
   return __builtin_bit_cast(h4, v);
 }
 
+// The same read, and a plain 16-byte read, at an LDS byte address (a 32-bit integer) plus a constant:
+// the constant travels in the instruction's immediate offset field.
+__device__ __forceinline__ h4 lds_read_tr_at(unsigned addr, int off) {
+  DA_LDS char* p = (DA_LDS char*)(unsigned long)addr + off;
+#ifdef DA_BF16
+  typedef short tr4i __attribute__((ext_vector_type(4)));
+  tr4i v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DA_LDS tr4i*)p);
+#else
+  tr4 v = __builtin_amdgcn_ds_read_tr16_b64_v4f16((DA_LDS tr4*)p);
+#endif
+  return __builtin_bit_cast(h4, v);
+}
+template <class V>
+__device__ __forceinline__ V lds_read_at(unsigned addr, int off) {
+  return *(const DA_LDS V*)((DA_LDS char*)(unsigned long)addr + off);
+}
+
 __device__ __forceinline__ h8 join(h4 lo, h4 hi) {
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
