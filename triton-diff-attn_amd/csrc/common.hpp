@@ -214,6 +214,7 @@ struct AsyncTile {
   }
   // number of instructions wave `wave` issues for one tile
   __device__ static __forceinline__ int count(int wave) {
+    if (NINST % NW == 0) return PER;   // the same for every wave: a compile-time constant
     int n = 0;
 #pragma unroll
     for (int k = 0; k < PER; ++k) n += (wave + NW * k < NINST) ? 1 : 0;

@@ -12,6 +12,8 @@
 //   * the P^T accumulator registers are reused directly (after fp16 packing) as the B operand of
 //     O^T = V^T * P^T; the V^T A-fragments come from the row-major V tile through the
 //     transposing LDS read, using the same key permutation as the accumulator layout.
+#include <type_traits>
+
 #include "params.hpp"
 
 namespace DA_NS {
@@ -30,7 +32,12 @@ struct FwdCfg {
   static constexpr int K_TILE = BN * D;            // halfs, one stream (swizzled, unpadded)
   static constexpr int V_TILE = BN * DV;
   static constexpr int K_BUF = 2 * K_TILE;         // K1 and K2 of one tile
-  static constexpr int NBUF = 3;                   // ring depth: tiles are fetched two iterations ahead
+  // Ring depth.  Tiles are fetched two iterations ahead, which takes three buffers; there are four so that
+  // the loop can be unrolled over one turn of the ring with every buffer known at compile time: an LDS
+  // address is then a per-lane register plus an immediate offset, with no arithmetic inside the loop.
+  static constexpr int NBUF = 4;
+  static constexpr int KBUF_BYTES = K_BUF * 2, VBUF_BYTES = V_TILE * 2, VBASE_BYTES = NBUF * KBUF_BYTES;
+  static_assert(NBUF * KBUF_BYTES <= 65536 && NBUF * VBUF_BYTES <= 65536, "immediate offsets reach every buffer");
   static constexpr int TILES = NBUF * (K_BUF + V_TILE);
   static constexpr int XCHG = NW * 32 * (DV + 8);            // halfs needed by the epilogue staging blocks
   static constexpr int SMEM = (TILES > XCHG) ? TILES : XCHG;
@@ -130,13 +137,33 @@ void fwd_kernel(FwdParams p) {
   auto load_va = [&](int tv, int buf) { VTile::template issue_at<0, VH>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n); };
   auto load_vb = [&](int tv, int buf) { VTile::template issue_at<VH, VTile::PER>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n); };
 
+  // Per-lane LDS byte addresses, computed once.  The XOR swizzle makes the address of a fragment a
+  // different function of the lane for every 16-byte chunk column, so there is one register per chunk
+  // column a lane reads; the ring buffer, the 32-key block and the k-step of 16 keys are multiples of 16
+  // rows, which the swizzle does not see, and travel in the instructions' immediate offsets.
+  // transposing-read coordinates of this lane inside a 16-key k-step: key row and feature column
+  const int tr_row = 4 * g + ((lane & 15) >> 2);
+  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const unsigned lds0 = (unsigned)(unsigned long)((DA_LDS char*)smem);
+  unsigned kb[NKS], vtr[NOT][2];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) kb[ks] = lds0 + 2u * (unsigned)(st * C::K_TILE + swz_off<D>(j, 16 * ks + 8 * g));
+#pragma unroll
+  for (int tt = 0; tt < NOT; ++tt)
+#pragma unroll
+    for (int e = 0; e < 2; ++e) vtr[tt][e] = lds0 + C::VBASE_BYTES + 2u * (unsigned)swz_off<DV>(tr_row + 8 * e, 32 * tt + tr_col);
+  // kept as they are: the compiler neither folds constants into them nor recomputes them in the loop
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) asm volatile("" : "+v"(kb[ks]));
+#pragma unroll
+  for (int tt = 0; tt < NOT; ++tt) asm volatile("" : "+v"(vtr[tt][0]), "+v"(vtr[tt][1]));
+
   // A-fragments of K for all k-steps of all 32-key tiles: row kt*32 + j, halfs 16ks + 8g .. +7
-  auto read_k = [&](const half_t* sK, h8 (&ka)[NKT][NKS]) {
+  auto read_k = [&](int byte_off, h8 (&ka)[NKT][NKS]) {
 #pragma unroll
     for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks)
-        ka[kt][ks] = *reinterpret_cast<const h8*>(sK + swz_off<D>(kt * 32 + j, 16 * ks + 8 * g));
+      for (int ks = 0; ks < NKS; ++ks) ka[kt][ks] = lds_read_at<h8>(kb[ks], byte_off + kt * 32 * D * 2);
   };
   auto scores = [&](const h8 (&ka)[NKT][NKS], f16v (&s)[QS][NKT]) {
 #pragma unroll
@@ -153,42 +180,45 @@ void fwd_kernel(FwdParams p) {
   const int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
   auto clampt = [&](int t) { return t < n_tiles ? t : n_tiles - 1; };   // past the end: harmless re-reads
 
+  // The loop below runs whole turns of the ring (NBUF iterations); the tile count is even, so when it is
+  // not a multiple of four, half a turn comes first and tile 0 goes into buffer 2: tile t is in buffer
+  // (t + b0) % NBUF, b0 = 0 or 2.
+  static_assert(C::NBUF == 4, "the loop is unrolled over a ring of four");
+  const bool head_half = (n_tiles & 2) != 0;
+  const int b0 = head_half ? 2 : 0;
   // prologue: K tiles 0..2 and V tiles 0..1; scores of tile 0
-  load_k1(0, 0); load_k2(0, 0); load_va(0, 0); load_vb(0, 0);
-  load_k1(clampt(1), 1); load_k2(clampt(1), 1); load_va(clampt(1), 1); load_vb(clampt(1), 1);
-  load_k1(clampt(2), 2); load_k2(clampt(2), 2);
+  load_k1(0, b0); load_k2(0, b0); load_va(0, b0); load_vb(0, b0);
+  load_k1(clampt(1), b0 + 1); load_k2(clampt(1), b0 + 1); load_va(clampt(1), b0 + 1); load_vb(clampt(1), b0 + 1);
+  load_k1(clampt(2), (b0 + 2) % 4); load_k2(clampt(2), (b0 + 2) % 4);
   wait_async_tiles();
   __syncthreads();
   f16v s_a[QS][NKT], s_b[QS][NKT];
   {
     h8 ka[NKT][NKS];
-    read_k(sKbuf + st * C::K_TILE, ka);
+    if (head_half) read_k(2 * C::KBUF_BYTES, ka);
+    else read_k(0, ka);
     scores(ka, s_a);
   }
-  __syncthreads();   // K buffer 0 is overwritten by the first iteration's prefetch
-  // ring positions: K tile t+1 is read from kb1, V tile t from vb0; K tile t+3 goes to kb0 (tile t,
-  // consumed one iteration ago), V tile t+2 to vb2 (tile t-1, likewise)
-  int kb0 = 0, kb1 = 1, vb0 = 0, vb2 = 2;
-  auto advance = [](int& b) { b = (b == 2) ? 0 : b + 1; };
-
-  // transposing-read coordinates of this lane inside a 16-key k-step: key row and feature column
-  const int tr_row = 4 * g + ((lane & 15) >> 2);
-  const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   // One iteration: softmax of tile t (scores in s_cur) and its P*V product, overlapped with the score
   // product of tile t+1 (into s_nxt).
-  auto iteration = [&](int t, f16v (&s_cur)[QS][NKT], f16v (&s_nxt)[QS][NKT]) {
+  // POS = (t + b0) % NBUF is the ring position: K tile t+1 is read from buffer POS+1 and V tile t from
+  // buffer POS; K tile t+3 goes to buffer POS+3 (tile t-1, consumed two iterations ago) and V tile t+2 to
+  // buffer POS+2 (tile t-2, likewise), all modulo NBUF.
+  auto iteration = [&](int t, auto pos_tag, f16v (&s_cur)[QS][NKT], f16v (&s_nxt)[QS][NKT]) {
+    constexpr int POS = decltype(pos_tag)::value;
+    constexpr int KR = (POS + 1) % 4, KP = (POS + 3) % 4, VR = POS, VP = (POS + 2) % 4;
     // Asynchronous prefetch straight into LDS, two iterations ahead: K tile t+3 and V tile t+2.
     // The groups of load instructions are spread over the iteration so that the waves do not
     // queue up behind each other at the memory pipeline.
     const int tk = clampt(t + 3);
     const int tv = clampt(t + 2);
-    load_k1(tk, kb0);
+    load_k1(tk, KP);
 
     // K fragments of the next tile are requested first; the row maxima of this tile are reduced
     // while they arrive.
     h8 ka[NKT][NKS];
-    read_k(sKbuf + kb1 * C::K_BUF + st * C::K_TILE, ka);
+    read_k(KR * C::KBUF_BYTES, ka);
 
     if constexpr (CAUSAL) {
       // only the last tiles of a wave's loop reach past its first row: mask key > query there
@@ -215,6 +245,12 @@ void fwd_kernel(FwdParams p) {
             if (kt * 32 + 8 * (r / 4) + (r % 4) > rel) s_cur[0][kt][r] = -INFINITY;
       }
     }
+
+    // The score product of the next tile goes to the matrix unit first and runs under the row maxima and
+    // the exponentials of this tile.  It starts from the running reference as it stands before this
+    // tile's update; when the update moves the reference, the few results are corrected with it.
+    load_k2(tk, KP);
+    scores(ka, s_nxt);
 
     float mx[QS];
 #pragma unroll
@@ -252,16 +288,14 @@ void fwd_kernel(FwdParams p) {
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) s_cur[qs][kt][r] -= d;
+          for (int r = 0; r < 16; ++r) { s_cur[qs][kt][r] -= d; s_nxt[qs][kt][r] -= d; }
 #pragma unroll
         for (int r = 0; r < 16; ++r) negm[qs][r] = -m[qs];
       }
     }
 
-    // From here on one basic block: the score product of the next tile and the P*V product of this
-    // tile run on the matrix unit while the exponentials run on the VALU.
-    load_k2(tk, kb0);
-    scores(ka, s_nxt);
+    // From here on one basic block: the P*V product of this tile runs on the matrix unit while the
+    // exponentials run on the VALU.
     // dropout: the mask arithmetic needs the registers of the K fragments, so the score product is
     // issued in full before the exponentials instead of between them
     if constexpr (DROP) __builtin_amdgcn_sched_barrier(0);
@@ -296,13 +330,12 @@ void fwd_kernel(FwdParams p) {
 
     // V^T fragments are requested PD products ahead of the product that uses them (measured: 2 and
     // 3 are 1.3 % faster than the single product the compiler picks by itself, 5 and 7 are not)
-    const half_t* sV = sVbuf + vb0 * C::V_TILE;
     constexpr int NPV = NKK * NOT;
     constexpr int PD = DROP ? 1 : 3;           // dropout: registers are short
     auto vt_frag = [&](int i) {
       const int kk = i / NOT, tt = i % NOT;
-      return join(lds_read_tr(sV + swz_off<DV>(16 * kk + tr_row, 32 * tt + tr_col)),
-                  lds_read_tr(sV + swz_off<DV>(16 * kk + 8 + tr_row, 32 * tt + tr_col)));
+      const int off = VR * C::VBUF_BYTES + 16 * kk * DV * 2;
+      return join(lds_read_tr_at(vtr[tt][0], off), lds_read_tr_at(vtr[tt][1], off));
     };
     h8 vfr[NPV];
 #pragma unroll
@@ -310,8 +343,8 @@ void fwd_kernel(FwdParams p) {
 #pragma unroll
     for (int i = 0; i < NPV; ++i) {
       const int kk = i / NOT, tt = i % NOT;
-      if (i == 0) load_va(tv, vb2);
-      if (i == NPV / 2) load_vb(tv, vb2);
+      if (i == 0) load_va(tv, VP);
+      if (i == NPV / 2) load_vb(tv, VP);
       if (i + PD < NPV) vfr[i + PD] = vt_frag(i + PD);
 #pragma unroll
       for (int qs = 0; qs < QS; ++qs) o[qs][tt] = mfma32(vfr[i], __builtin_bit_cast(h8, pw[qs][kk]), o[qs][tt]);
@@ -320,13 +353,21 @@ void fwd_kernel(FwdParams p) {
     // the tiles needed next were requested one iteration ago: only this iteration's loads may remain
     wait_async_tiles_except(loads_per_iter);
     __syncthreads();
-    advance(kb0); advance(kb1); advance(vb0); advance(vb2);
   };
 
   // the tile count is even (N is a multiple of 128, tiles are at most 64 keys)
-  for (int t = 0; t < n_tiles; t += 2) {
-    iteration(t, s_a, s_b);
-    iteration(t + 1, s_b, s_a);
+  int t = 0;
+  if (head_half) {
+    iteration(0, std::integral_constant<int, 2>{}, s_a, s_b);
+    iteration(1, std::integral_constant<int, 3>{}, s_b, s_a);
+    t = 2;
+  }
+#pragma nounroll
+  for (; t < n_tiles; t += 4) {
+    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b);
+    iteration(t + 1, std::integral_constant<int, 1>{}, s_b, s_a);
+    iteration(t + 2, std::integral_constant<int, 2>{}, s_a, s_b);
+    iteration(t + 3, std::integral_constant<int, 3>{}, s_b, s_a);
   }
 
   wait_async_tiles();   // the staging blocks below reuse the tile memory the last prefetches write to
