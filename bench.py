@@ -22,7 +22,6 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "triton-diff-attn_amd"))
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 PEAK_FP16_TFLOPS = 2500.0     # MI355X published dense fp16 MFMA peak (2.5 PFLOP/s)
 
@@ -32,6 +31,14 @@ WORKLOADS = {
     "config4": dict(B=8, H=32, N=4096, D=128, lam=0.8, lambda_init=0.2, rms=False, seed=4, scale=1.0),
     # the headline shape with the causal mask (an addition to the reference's operator)
     "headline_causal": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0, causal=True),
+    # the operator's additions to the reference, at the headline shape: what each costs against "headline"
+    "headline_bf16": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0, bf16=True),
+    "headline_dropout": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0, dropout=0.1),
+    "headline_per_head": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0, per_head=True),
+    # q/k/v as views of token-major [B,N,H,.] buffers (a projection's output), read through their strides
+    "headline_token_major": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0, token_major=True),
+    # a sequence length that is not a multiple of the kernels' 128-row blocks
+    "headline_ragged": dict(B=4, H=32, N=2000, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0),
     # forward-only configurations: a step is one forward without gradients
     "config0": dict(B=2, H=16, N=512, D=32, lam=0.5, lambda_init=0.8, rms=True, seed=0, scale=1.0, fwd_only=True),
     "headline_fwd": dict(B=4, H=32, N=2048, D=64, lam=0.5, lambda_init=0.8, rms=True, seed=2, scale=1.0, fwd_only=True),
@@ -98,7 +105,7 @@ def gpu_max_clock_mhz(torch):
 def cpu_baseline(cfg, torch, budget_s=12.0):
     """Times the fp32 oracle (forward + autograd backward) on a few (b,h) units of the workload."""
     from oracle import diff_attn_oracle as orc
-    from util import make_inputs
+    from synthetic import make_inputs
 
     cores = os.cpu_count() or 1
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
@@ -148,7 +155,7 @@ def main():
     import torch
     import _native
     from layers import MultiheadDiffAttnKernel
-    from util import make_inputs
+    from synthetic import make_inputs
 
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
@@ -158,21 +165,29 @@ def main():
     prop = torch.cuda.get_device_properties(0)
     lib = _native.lib()
 
-    q1, q2, k1, k2, v, dy = (t.to(dev) for t in make_inputs(B, H, N, D, cfg["seed"], cfg["scale"]))
+    dtype = torch.bfloat16 if cfg.get("bf16") else torch.float16
+    q1, q2, k1, k2, v, dy = (t.to(dev).to(dtype) for t in make_inputs(B, H, N, D, cfg["seed"], cfg["scale"]))
+    if cfg.get("token_major"):
+        # the same values in [B,N,H,.] memory, seen as [B,H,N,.]
+        q1, q2, k1, k2, v = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q1, q2, k1, k2, v))
     fwd_only = bool(cfg.get("fwd_only"))
     leaves = [t.requires_grad_(not fwd_only) for t in (q1, q2, k1, k2, v)]
-    lam = torch.tensor([cfg["lam"]], dtype=torch.float16, device=dev, requires_grad=not fwd_only)
+    lam = torch.tensor([cfg["lam"]] * (H if cfg.get("per_head") else 1), dtype=dtype, device=dev, requires_grad=not fwd_only)
+    extra = {}
+    if cfg.get("causal"):
+        extra["causal"] = True
+    if cfg.get("dropout"):
+        extra.update(dropout_p=cfg["dropout"], dropout_seed=1234)
 
     def step():
         if fwd_only:
             with torch.no_grad():
-                MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"])
+                MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"], **extra)
             return
         for t in leaves:
             t.grad = None
         lam.grad = None
-        y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"],
-                                    causal=bool(cfg.get("causal")))
+        y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"], **extra)
         y.backward(dy)
 
     if args.graph:
@@ -192,10 +207,10 @@ def main():
         with torch.cuda.graph(whole):
             if fwd_only:
                 with torch.no_grad():
-                    MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"])
+                    MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"], **extra)
             else:
                 MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=cfg["lambda_init"], rms_norm=cfg["rms"],
-                                        causal=bool(cfg.get("causal"))).backward(dy)
+                                        **extra).backward(dy)
 
         def step():      # noqa: F811  (replaces the eager step)
             whole.replay()
@@ -215,29 +230,40 @@ def main():
 
     # ---- per-kernel timings through the C ABI, events on the launch stream ----
     with torch.no_grad():
-        yb = torch.empty_like(v); u2 = torch.empty_like(v)
-        lse1 = torch.empty(B, H, N, device=dev); lse2 = torch.empty(B, H, N, device=dev)
-        rinv = torch.empty(B, H, N, device=dev)
-        grads = [torch.empty_like(t) for t in (q1, q2, k1, k2, v)]
-        dlam = torch.empty(1, dtype=torch.float16, device=dev)
-        flags = int(cfg["rms"]) | (2 if cfg.get("causal") else 0)     # DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL
-        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D, flags)
+        n_pad = -(-N // 128) * 128
+        # a length that is not a multiple of 128 runs on the next one inside the kernels; only the library's own
+        # buffers (u2, the row statistics, the workspace) have the padded length
+        kq1, kq2, kk1, kk2, kv, kdy = q1, q2, k1, k2, v, dy
+        yb = torch.empty_like(kv); u2 = torch.empty(B, H, n_pad, 2 * D, device=dev, dtype=dtype)
+        lse1 = torch.empty(B, H, n_pad, device=dev); lse2 = torch.empty(B, H, n_pad, device=dev)
+        rinv = torch.empty(B, H, n_pad, device=dev)
+        grads = [torch.empty_like(t) for t in (kq1, kq2, kk1, kk2, kv)]      # in the layout of their tensors
+        dlam = torch.empty(lam.numel(), dtype=dtype, device=dev)
+        # DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL | DIFFATTN_BF16 | DIFFATTN_LAMBDA_PER_HEAD | DIFFATTN_UNPADDED
+        flags = (int(cfg["rms"]) | (2 if cfg.get("causal") else 0) | (4 if cfg.get("bf16") else 0)
+                 | (8 if cfg.get("per_head") else 0) | (32 if n_pad != N else 0))
+        layout = None
+        if cfg.get("token_major"):
+            layout = _native.Layout(*kq1.stride()[:3], *kv.stride()[:3], *yb.stride()[:3], *kdy.stride()[:3],
+                                    *grads[0].stride()[:3], *grads[4].stride()[:3])
+        drop = _native.Dropout(cfg["dropout"], 1234) if cfg.get("dropout") else None
+        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, n_pad, D, flags)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         stream = torch.cuda.current_stream().cuda_stream
         sm = 1 / math.sqrt(D)
 
         def launch_forward():
-            _native.check(lib.diffattn_forward(
-                q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
+            _native.check(lib.diffattn_forward_padded(
+                kq1.data_ptr(), kq2.data_ptr(), kk1.data_ptr(), kk2.data_ptr(), kv.data_ptr(), lam.data_ptr(),
                 yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(),
-                B, H, N, D, sm, cfg["lambda_init"], flags, stream))
+                B, H, n_pad, N, D, sm, cfg["lambda_init"], flags, layout, drop, stream))
 
         def bwd_stage(mask):
             return lambda: _native.check(lib.diffattn_backward_stages(
-                q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
-                yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(), dy.data_ptr(),
+                kq1.data_ptr(), kq2.data_ptr(), kk1.data_ptr(), kk2.data_ptr(), kv.data_ptr(), lam.data_ptr(),
+                yb.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), rinv.data_ptr(), kdy.data_ptr(),
                 *[g.data_ptr() for g in grads], dlam.data_ptr(), ws.data_ptr(), ws_bytes,
-                B, H, N, N, D, sm, cfg["lambda_init"], flags, mask, None, None, stream))
+                B, H, n_pad, N, D, sm, cfg["lambda_init"], flags, mask, layout, drop, stream))
 
         launch_forward()
         k_iters = max(5, min(args.steps, 30))
@@ -255,27 +281,34 @@ def main():
     # in a forward-only workload the forward kernel with its 12*B*H*N^2*D
     dom, dom_flops = ("fwd_kernel", 12 * unit) if fwd_only else ("bwd_dkdv_kernel", 16 * unit)
     dom_tflops = dom_flops / (kernels_ms[dom] * 1e-3) / 1e12
-    traffic = None
+    # HBM bytes per launch are not measured in this run: they are read from the committed summary of two
+    # rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of this workload, when there is one (see the file's note)
+    traffic = traffic_source = None
     tpath = os.path.join(ROOT, "profiles", "traffic_%s.json" % args.workload)
     if os.path.exists(tpath):
-        # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the file's note)
         k = json.load(open(tpath))["kernels"].get(dom)
-        traffic = k["fetch_bytes"] + k["write_bytes"] if k else None
+        if k:
+            traffic = k["fetch_bytes"] + k["write_bytes"]
+            traffic_source = "profiles/traffic_%s.json (static: rocprofv3 --pmc summary, not measured in this run)" % args.workload
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": dom_tflops, "peak": PEAK_FP16_TFLOPS,
         "unit": "TFLOP/s", "frac": dom_tflops / PEAK_FP16_TFLOPS, "traffic": traffic,
-        "flops_per_launch": dom_flops, "ms_per_launch": kernels_ms[dom],
+        "traffic_source": traffic_source, "flops_per_launch": dom_flops, "ms_per_launch": kernels_ms[dom],
     }
 
     out = {
         "metric": "fwd+bwd TFLOP/s & % fp16 MFMA peak, diff-attn B4 H32 N2048 D64",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "%s: diff-attn %s B%d H%d N%d D%d fp16 rms_norm=%s lambda=%.1f lambda_init=%.1f"
+        "dtype": "bf16" if cfg.get("bf16") else "f16", "data": "synthetic",
+        "config": {"workload": "%s: diff-attn %s B%d H%d N%d D%d rms_norm=%s lambda=%.1f lambda_init=%.1f"
                                % (args.workload, "fwd" if fwd_only else "fwd+bwd", B, H, N, D, cfg["rms"], cfg["lam"],
                                   cfg["lambda_init"])
-                               + (" causal" if cfg.get("causal") else "") + (" (HIP graph replay)" if args.graph else "")},
+                               + (" causal" if cfg.get("causal") else "") + (" bf16" if cfg.get("bf16") else "")
+                               + (" dropout=%.2f" % cfg["dropout"] if cfg.get("dropout") else "")
+                               + (" one lambda per head" if cfg.get("per_head") else "")
+                               + (" token-major q/k/v read through strides" if cfg.get("token_major") else "")
+                               + (" (HIP graph replay)" if args.graph else "")},
         "frac_of_fp16_mfma_peak": value / PEAK_FP16_TFLOPS,
         # the K timed steps one by one (an event between steps): median and the 5 % / 95 % quantiles
         "ms_per_step_median": quantile(per_step, 0.5), "ms_per_step_p5": quantile(per_step, 0.05),

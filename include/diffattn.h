@@ -12,7 +12,7 @@
  *     gradients, [B,H,N,2D] for v, y, u2, dy, dv; row statistics are fp32 [B,H,N];
  *   - D is 32, 64 or 128; N is a multiple of 128;
  *   - lambda_scale is a DEVICE pointer to one fp16 value (the reference loads it in-kernel,
- *     src/kernel.py:138), or to H values with DIFFATTN_LAMBDA_PER_HEAD;
+ *     src/kernel.py:138), or to H values with DIFFATTN_LAMBDA_PER_HEAD; fp32 values with DIFFATTN_LAMBDA_FP32;
  *   - `stream` is a hipStream_t passed as void*; work is only enqueued on it.  No entry point
  *     allocates, frees, synchronises or keeps global state; all are re-entrant;
  *   - return value: 0 on success, a negative DIFFATTN_E* code for rejected arguments, or a
@@ -35,8 +35,8 @@ extern "C" {
 #define DIFFATTN_EINVAL_ALIGN (-5)  /* a pointer is not 16-byte aligned */
 #define DIFFATTN_EINVAL_FLAGS (-6)  /* unknown bits in `flags` */
 #define DIFFATTN_EINVAL_SCRATCH (-7) /* problem too large for diffattn_backward_static */
+#define DIFFATTN_EINVAL_LAYOUT (-8)  /* a stride in diffattn_layout is negative, not a multiple of 8, a row stride is below the row width, or y overlaps itself */
 #define DIFFATTN_EINVAL_DROPOUT (-9) /* dropout probability outside [0, 255/256] */
-#define DIFFATTN_EINVAL_LAYOUT (-8)  /* a stride in diffattn_layout is negative, not a multiple of 8, or a row stride is below the row width */
 
 /* `flags` of the forward and backward entry points.  DIFFATTN_RMS_NORM is the reference's boolean
  * `rms_norm` (src/kernel.py:464): a caller that passes a C boolean there keeps working.
@@ -52,6 +52,16 @@ extern "C" {
  * the backward writes H values to dlambda, each summed over the batch.  No counterpart in the
  * reference, which has one lambda per call (src/kernel.py:138). */
 #define DIFFATTN_LAMBDA_PER_HEAD 8
+/* *lambda_scale is read and *dlambda is written as fp32, whatever the type of the tensors.  The reference
+ * returns the lambda gradient in the tensors' fp16 (`dtype=V.dtype`, src/kernel.py:573), where it
+ * saturates at 65504: under a gradient scaler's loss scale the sum over all rows reaches that quickly.
+ * With this flag the fixed-order fp32 sum leaves the library unrounded. */
+#define DIFFATTN_LAMBDA_FP32 16
+/* The caller's tensors (q1, q2, k1, k2, v, y, dy and the gradients) hold n_valid rows per (batch, head)
+ * unit instead of N: a dense one is [B,H,n_valid,C].  See diffattn_forward_padded.  Without the flag a
+ * dense tensor is [B,H,N,C] (the caller has padded it); either way no row past n_valid-1 of those
+ * tensors is read or written. */
+#define DIFFATTN_UNPADDED 32
 
 /*
  * Element strides of the caller's tensors, for the entry points that take a `layout`.  The
@@ -60,15 +70,21 @@ extern "C" {
  * their own.  Each tensor is logically [B,H,N,C] with the last dimension contiguous; `_b`, `_h`,
  * `_n` are the distances in elements between batch entries, heads and rows.  Every stride must be
  * a non-negative multiple of 8 (rows start 16-byte aligned) and a row stride at least C; a
- * [B,N,H,C] buffer viewed as [B,H,N,C] is `{N*H*C, C, H*C}`.  Everything the library writes for
- * itself or returns as a gradient (u2, the row statistics, dq1, dq2, dk1, dk2, dv) stays dense.
- * A NULL `layout` means every tensor is dense.
+ * [B,N,H,C] buffer viewed as [B,H,N,C] is `{N*H*C, C, H*C}`.  A zero batch or head stride broadcasts an
+ * input; a tensor that is written (y, the gradients) must not overlap itself (non-zero batch and head
+ * strides when B, H > 1).  The gradients have strides of their own, so that they can be written in the
+ * layout of the tensors they belong to (dq1, dq2, dk1, dk2 share one set, like q1..k2); all three zero
+ * means dense.  What the library writes for itself (u2, the row statistics, the workspace) is dense
+ * [B,H,N,.].  A NULL `layout` means every tensor is dense.
  */
 typedef struct diffattn_layout {
   long long qk_b, qk_h, qk_n;   /* q1, q2, k1, k2  (C = D)  */
   long long v_b, v_h, v_n;      /* v               (C = 2D) */
   long long y_b, y_h, y_n;      /* y               (C = 2D) */
-  long long dy_b, dy_h, dy_n;   /* dy, backward only (C = 2D); ignored by the forward */
+  /* backward only; the forward neither reads nor checks these */
+  long long dy_b, dy_h, dy_n;       /* dy                  (C = 2D) */
+  long long dqk_b, dqk_h, dqk_n;    /* dq1, dq2, dk1, dk2  (C = D); all zero: dense  */
+  long long dv_b, dv_h, dv_n;       /* dv                  (C = 2D); all zero: dense */
 } diffattn_layout;
 
 /*
@@ -111,13 +127,15 @@ int diffattn_forward(const void* q1, const void* q2, const void* k1, const void*
 
 /*
  * Forward for a sequence whose real length n_valid is not a multiple of 128.  No counterpart in the
- * reference, whose kernels require such a multiple (src/kernel.py:4, :527).  The caller pads every
- * tensor with zero rows to N (a multiple of 128, n_valid <= N); keys n_valid..N-1 are ignored, rows
- * n_valid..N-1 of the outputs are to be discarded.  The matching backward is
- * diffattn_backward_stages with the same n_valid, on the padded tensors with zero rows of dy in the
- * padding; it returns the gradients of rows 0..n_valid-1.  diffattn_forward is this function with
- * n_valid = N.  `layout` gives the strides of q1, q2, k1, k2, v and y (NULL: all dense);
- * `dropout` switches dropout on (NULL: none).
+ * reference, whose kernels require such a multiple and have no boundary checks (src/kernel.py:4,
+ * :136-150, :527).  N is n_valid rounded up to a multiple of 128: the kernels work on N rows, u2, lse1,
+ * lse2 and rinv have N rows per unit, and so has the backward's workspace.  Of q1, q2, k1, k2, v and y only
+ * rows 0..n_valid-1 are touched: reads past them are redirected to the last real row inside the kernels,
+ * keys n_valid..N-1 are ignored, and y gets no rows past n_valid-1.  So the caller's tensors need only
+ * n_valid rows (say so with DIFFATTN_UNPADDED, or pass their strides in `layout`); tensors padded to N rows
+ * by the caller work as well.  The matching backward is diffattn_backward_stages with the same N, n_valid
+ * and flags.  diffattn_forward is this function with n_valid = N.  `layout` gives the strides of q1, q2,
+ * k1, k2, v and y (NULL: all dense); `dropout` switches dropout on (NULL: none).
  */
 int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, const void* k2, const void* v,
                             const void* lambda_scale, void* y, void* u2, float* lse1, float* lse2, float* rinv,
@@ -135,8 +153,8 @@ size_t diffattn_backward_workspace_bytes(int B, int H, int N, int D, int flags);
  *   inputs : q1,q2,k1,k2,v,lambda_scale as in forward; y,u2,lse1,lse2,rinv as written by forward
  *            (rinv is ignored without DIFFATTN_RMS_NORM); dy [B,H,N,2D] upstream gradient, dense.
  *   outputs: dq1,dq2,dk1,dk2 [B,H,N,D], dv [B,H,N,2D] fp16; dlambda: one fp16 value (H values
- *            with DIFFATTN_LAMBDA_PER_HEAD), DEVICE memory, written (not accumulated), reduced in
- *            a fixed order: bit-reproducible.
+ *            with DIFFATTN_LAMBDA_PER_HEAD; fp32 with DIFFATTN_LAMBDA_FP32), DEVICE memory, written
+ *            (not accumulated), reduced in a fixed order: bit-reproducible.
  *   workspace: device memory of at least diffattn_backward_workspace_bytes(B,H,N,D,flags) bytes,
  *            256-byte aligned, contents undefined before and after.
  */
@@ -162,9 +180,10 @@ int diffattn_backward(const void* q1, const void* q2, const void* k1, const void
  * The outputs of a stage that is not requested may be NULL: a caller that needs, say, only dQ1 and
  * dQ2 passes PREP | DQ and NULL for dk1, dk2, dv and dlambda.
  * n_valid (1..N) is the real sequence length of a problem that went through
- * diffattn_forward_padded (N when there is no padding): keys n_valid..N-1 are ignored.
- * `layout` gives the strides of q1, q2, k1, k2, v, y and dy (NULL: all dense); the gradients are
- * written dense.  `dropout` must be what the forward was given.
+ * diffattn_forward_padded (N when there is no padding): keys n_valid..N-1 are ignored, rows
+ * n_valid..N-1 of q1, q2, k1, k2, v, y and dy are not read and those of the gradients not written.
+ * `layout` gives the strides of q1, q2, k1, k2, v, y, dy and of the gradients (NULL: all dense).
+ * `dropout` must be what the forward was given.
  */
 #define DIFFATTN_STAGE_PREP 1u
 #define DIFFATTN_STAGE_DLAMBDA 2u

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared_symbols():
         assert hasattr(lib, name), name
         assert name in _native.SYMBOLS, "binding table misses %s" % name
-    assert lib.diffattn_abi_version() == 6 == _native.ABI_VERSION
+    assert lib.diffattn_abi_version() == 7 == _native.ABI_VERSION
 
 
 def test_argument_rejection_needs_no_gpu():
@@ -72,8 +72,26 @@ def test_argument_rejection_needs_no_gpu():
                 y_b=128 * 128, y_h=128, y_n=128, dy_b=128 * 128, dy_h=128, dy_n=128)
     for field, value in (("qk_n", 32), ("v_n", 132), ("y_h", -8), ("dy_b", 4)):
         lay = _native.Layout(**dict(good, **{field: value}))
-        assert lib.diffattn_forward_padded(*padded(128, ctypes.byref(lay))) == -8, field
+        if not field.startswith("dy"):
+            assert lib.diffattn_forward_padded(*padded(128, ctypes.byref(lay))) == -8, field
         assert lib.diffattn_backward_stages(*sargs(256, ctypes.byref(lay))) == -8, field
+    # y, which is written, may not overlap itself
+    padded2 = lambda layout: [p] * 11 + [2, 2, 128, 128, 64, 0.125, 0.8, 1, layout, None, None]
+    for field in ("y_b", "y_h"):
+        lay = _native.Layout(**dict(good, **{field: 0}))
+        assert lib.diffattn_forward_padded(*padded2(ctypes.byref(lay))) == -8, field
+    # Arguments that pass validation reach the launch, which fails with a positive HIP error code where there
+    # is no GPU; the pointers here are host memory, so these calls are made only where nothing can run.
+    if not torch.cuda.is_available():
+        # the forward neither reads nor checks the strides of dy: a forward-only caller may leave them zero
+        fwd_only = _native.Layout(**{k: (0 if k.startswith("dy") else v) for k, v in good.items()})
+        assert lib.diffattn_forward_padded(*padded(128, ctypes.byref(fwd_only))) > 0
+        assert lib.diffattn_forward_padded(*padded(128, ctypes.byref(_native.Layout(**dict(good, dy_b=4))))) > 0
+        broadcast_v = _native.Layout(**dict(good, v_b=0))       # an input may be broadcast over the batch
+        assert lib.diffattn_forward_padded(*padded2(ctypes.byref(broadcast_v))) > 0
+        lam32 = padded(128)
+        lam32[18] = 1 | 16                                      # DIFFATTN_RMS_NORM | DIFFATTN_LAMBDA_FP32
+        assert lib.diffattn_forward_padded(*lam32) > 0
     for bad_p in (-0.1, 1.0, float("nan")):
         drop = _native.Dropout(bad_p, 1)
         assert lib.diffattn_forward_padded(*padded(128, None, ctypes.byref(drop))) == -9, bad_p
@@ -103,8 +121,12 @@ def test_host_validation_errors():
         _lambda_tensor(torch.zeros(2), torch.device("cpu"))
     with pytest.raises(ValueError):   # neither one value nor one per head
         _lambda_tensor(torch.zeros(3), torch.device("cpu"), num_heads=4)
-    per_head = _lambda_tensor(torch.tensor([[0.1], [0.2], [0.3]]), torch.device("cpu"), num_heads=3)
+    per_head = _lambda_tensor(torch.tensor([[0.1], [0.2], [0.3]], dtype=torch.float16), torch.device("cpu"), num_heads=3)
     assert per_head.shape == (3,) and per_head.dtype == torch.float16
+    # an fp32 lambda is read as fp32 (and gets an fp32 gradient); other types go through the tensors' dtype
+    assert _lambda_tensor(torch.tensor([[0.1], [0.2], [0.3]]), torch.device("cpu"), num_heads=3).dtype == torch.float32
+    assert _lambda_tensor(torch.tensor([0.5], dtype=torch.float64), torch.device("cpu"), torch.bfloat16).dtype == torch.bfloat16
+    assert _lambda_tensor(0.5, torch.device("cpu"), torch.bfloat16).dtype == torch.bfloat16
     from kernel import _pad_rows
     x = torch.arange(2 * 3 * 5 * 4, dtype=torch.float16).reshape(2, 3, 5, 4)
     padded = _pad_rows(x, 8)

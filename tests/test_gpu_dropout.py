@@ -84,3 +84,39 @@ def test_zero_probability_is_the_plain_operator():
     assert torch.equal(plain, zero)
     with pytest.raises(ValueError):
         MultiheadDiffAttnKernel(q1, q2, k1, k2, v, lam, 0.8, True, dropout_p=1.0)
+
+
+def test_mask_dump_equals_the_host_model_of_the_hash():
+    """Bit for bit: the library's keep decisions against tests/dropout_model.py, whose statistics the CPU
+    tests check (keep rate, independence across seeds, units and streams)."""
+    import numpy as np
+    import dropout_model as dm
+    B, H, N, p = 2, 3, 128, 0.25
+    for seed in (0, 1, 0x1234_5678_9ABC_DEF0):
+        m1, m2 = kernel_masks(B, H, N, p, seed)
+        for unit in (0, 1, B * H - 1):
+            b, h = divmod(unit, H)
+            assert np.array_equal(m1[b, h].numpy(), dm.keep_mask(seed, unit, 0, N, p)), (seed, unit, 0)
+            assert np.array_equal(m2[b, h].numpy(), dm.keep_mask(seed, unit, 1, N, p)), (seed, unit, 1)
+
+
+def test_dropout_under_stream_capture_needs_a_seed():
+    from layers import MultiheadDiffAttnKernel
+    cpu = make_inputs(1, 2, 128, 64, seed=5)
+    t = [x.cuda() for x in cpu[:5]]
+    lam = torch.tensor([0.5], dtype=torch.float16, device="cuda")
+    MultiheadDiffAttnKernel(*t, lambda_scale=lam, dropout_p=0.1)       # eager: a seed is drawn
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        MultiheadDiffAttnKernel(*t, lambda_scale=lam, dropout_p=0.1, dropout_seed=3)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        with pytest.raises(RuntimeError, match="explicit dropout_seed"):
+            MultiheadDiffAttnKernel(*t, lambda_scale=lam, dropout_p=0.1)
+        y = MultiheadDiffAttnKernel(*t, lambda_scale=lam, dropout_p=0.1, dropout_seed=3)     # a named seed is fine
+    g.replay()
+    torch.cuda.synchronize()
+    assert torch.isfinite(y).all()

@@ -1,6 +1,7 @@
-"""Sequence lengths that are not multiples of 128 (a restriction of the reference's kernels, src/kernel.py:4,
-:527): the host pads, the forward ignores the padding keys, the backward is exact on the real rows.
-Checked against the fp32 oracle at the unpadded length, with the tolerances of the other parity tests."""
+"""Sequence lengths that are not multiples of 128 (a restriction of the reference's kernels, which have no
+boundary checks, src/kernel.py:4, :136-150, :527): the kernels run on the next multiple of 128, never touch a
+row of the caller's tensors past the real length, and ignore the padding keys; nothing is padded or copied on
+the host.  Checked against the fp32 oracle at the real length, with the tolerances of the other parity tests."""
 import pytest
 import torch
 
@@ -66,3 +67,67 @@ def test_padding_does_not_leak_into_real_rows():
     views = [t[:, :, :200] for t in (q1, q2, k1, k2, v)]                  # non-contiguous views of longer tensors
     y_b, g_b = run_kernel(*views, 0.5, 0.8, True, dy[:, :, :200])
     assert torch.equal(y_a, y_b) and all(torch.equal(a, b) for a, b in zip(g_a, g_b))
+
+
+@pytest.mark.parametrize("D,n_valid,causal,rms", [(64, 200, False, True), (32, 130, True, True), (128, 255, False, False),
+                                                   (64, 70, True, False), (64, 129, False, True)])
+def test_rows_past_the_real_length_are_neither_read_nor_written(D, n_valid, causal, rms):
+    """Through the C ABI, on buffers of the padded length: input rows past n_valid hold NaN (a kernel that read
+    them would spread it), output rows past n_valid hold a sentinel (a kernel that wrote them would erase it)."""
+    import math
+    import _native
+    lib = _native.lib()
+    B, H, N = 2, 3, 256
+    cpu = make_inputs(B, H, N, D, seed=35)
+    dev = [t.cuda() for t in cpu]
+    for t in dev:
+        t[:, :, n_valid:] = float("nan")
+    q1, q2, k1, k2, v, dy = dev
+    lam = torch.tensor([0.5], dtype=torch.float16, device="cuda")
+    sentinel = 777.0
+    y = torch.full_like(v, sentinel)
+    u2 = torch.empty_like(v)
+    lse1, lse2, rinv = (torch.empty(B, H, N, device="cuda") for _ in range(3))
+    grads = [torch.full_like(t, sentinel) for t in (q1, q2, k1, k2, v)]
+    dlam = torch.empty(1, dtype=torch.float16, device="cuda")
+    flags = (1 if rms else 0) | (2 if causal else 0)
+    ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D, flags)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    sm = 1 / math.sqrt(D)
+    _native.check(lib.diffattn_forward_padded(q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
+                                              lam.data_ptr(), y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(),
+                                              rinv.data_ptr(), B, H, N, n_valid, D, sm, 0.8, flags, None, None, st))
+    _native.check(lib.diffattn_backward_stages(q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(),
+                                               lam.data_ptr(), y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(),
+                                               rinv.data_ptr(), dy.data_ptr(), *[g.data_ptr() for g in grads], dlam.data_ptr(),
+                                               ws.data_ptr(), ws_bytes, B, H, N, n_valid, D, sm, 0.8, flags, 15, None, None, st))
+    torch.cuda.synchronize()
+    cut = [t[:, :, :n_valid].contiguous() for t in cpu]
+    ref = orc.forward_backward(*cut[:5], torch.tensor([0.5], dtype=torch.float16), cut[5], 0.8, rms, chunk=1, causal=causal)
+    assert (y[:, :, n_valid:] == sentinel).all() and all((g[:, :, n_valid:] == sentinel).all() for g in grads)
+    assert max_abs(y[:, :, :n_valid], ref[0]) <= Y_ATOL
+    for name, g, r in zip(("dq1", "dq2", "dk1", "dk2", "dv"), grads, ref[1:6]):
+        assert torch.isfinite(g[:, :, :n_valid]).all(), name
+        assert rel_to_max(g[:, :, :n_valid], r) <= GRAD_RTOL, name
+    assert rel_to_max(dlam, ref[6]) <= GRAD_RTOL
+
+
+def test_nothing_is_copied_for_a_ragged_length():
+    """The operator hands the caller's tensors to the kernels as they are: the output and the gradients have the
+    real length, and the gradients of token-major views come back in that layout."""
+    from layers import MultiheadDiffAttnKernel
+    B, H, N, D = 2, 4, 200, 64
+    cpu = make_inputs(B, H, N, D, seed=36)
+    # [B,N,H,.] buffers seen as [B,H,N,.]
+    leaves = [t.cuda().transpose(1, 2).contiguous().transpose(1, 2).requires_grad_(True) for t in cpu[:5]]
+    lam = torch.tensor([0.5], dtype=torch.float16, device="cuda", requires_grad=True)
+    y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam, lambda_init=0.8, rms_norm=True)
+    assert y.shape == (B, H, N, 2 * D) and y.stride() == leaves[4].stride()
+    y.backward(cpu[5].cuda())
+    torch.cuda.synchronize()
+    assert all(t.grad.shape == t.shape and t.grad.stride() == t.stride() for t in leaves)
+    ref = orc.forward_backward(*cpu[:5], torch.tensor([0.5], dtype=torch.float16), cpu[5], 0.8, True, chunk=1)
+    assert max_abs(y, ref[0]) <= Y_ATOL
+    for name, t, r in zip(("dq1", "dq2", "dk1", "dk2", "dv"), leaves, ref[1:6]):
+        assert rel_to_max(t.grad, r) <= GRAD_RTOL, name

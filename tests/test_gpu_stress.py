@@ -62,3 +62,29 @@ def test_upstream_gradient_with_a_loss_scale(D, scale):
     for name, g, r in zip(("dq1", "dq2", "dk1", "dk2", "dv"), grads, ref[1:6]):
         assert torch.isfinite(g).all(), name
         assert rel_to_max(g.float() / scale, r) <= GRAD_RTOL, name
+
+
+@pytest.mark.parametrize("D", [32, 64])
+def test_lambda_gradient_under_a_loss_scale(D):
+    """The lambda gradient sums over every row of every unit, so it leaves the fp16 range long before the
+    other gradients do.  With lambda in fp32 the library reads it and returns its gradient in fp32: exact up
+    to the usual tolerance whatever the loss scale.  With lambda in fp16 the gradient is rounded to fp16 as
+    the reference's is (src/kernel.py:573) and saturates to infinity beyond 65504."""
+    from layers import MultiheadDiffAttnKernel
+    B, H, N, scale = 2, 4, 1024, 1024.0
+    q1, q2, k1, k2, v, dy = make_inputs(B, H, N, D, seed=47)
+    ref = orc.forward_backward(q1, q2, k1, k2, v, torch.tensor([0.5], dtype=torch.float16), dy, 0.8, True)
+    want = ref[6].float().item() * scale
+    assert abs(want) > 65504, "the case is meant to leave the fp16 range (got %g)" % want
+    got = {}
+    for dtype in (torch.float32, torch.float16):
+        t = [x.cuda().requires_grad_(True) for x in (q1, q2, k1, k2, v)]
+        lam = torch.tensor([0.5], dtype=dtype, device="cuda", requires_grad=True)
+        y = MultiheadDiffAttnKernel(*t, lambda_scale=lam, lambda_init=0.8, rms_norm=True)
+        y.backward((dy * scale).half().cuda())
+        assert lam.grad.dtype == dtype and lam.grad.shape == lam.shape
+        got[dtype] = lam.grad.float().item()
+        for name, g, r in zip(("dq1", "dq2", "dk1", "dk2", "dv"), (x.grad for x in t), ref[1:6]):
+            assert rel_to_max(g.float().cpu() / scale, r) <= GRAD_RTOL, name
+    assert abs(got[torch.float32] - want) <= GRAD_RTOL * abs(want)
+    assert got[torch.float16] == float("inf") * (1 if want > 0 else -1)      # the documented saturation

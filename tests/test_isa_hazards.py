@@ -79,3 +79,21 @@ def test_forward_kernels_do_not_spill_in_their_loops(tmp_path):
             m = re.match(r"\s+s_cbranch_\w+ (\.LBB\w+)", l)
             if m and label_at.get(m.group(1), i) < i:
                 assert not any("scratch_" in x for x in lines[label_at[m.group(1)]:i]), name
+
+
+def test_build_rejects_a_spilling_kernel():
+    """build.py reads the compiler's per-kernel resource remarks and refuses kernels that must not spill."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("da_build", os.path.join(ROOT, "triton-diff-attn_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    remark = ("x.hip:1:1: remark: Function Name: %s [-Rpass-analysis=kernel-resource-usage]\n"
+              "x.hip:1:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]\n"
+              "x.hip:1:1: remark:     ScratchSize [bytes/lane]: %d [-Rpass-analysis=kernel-resource-usage]\n")
+    dkdv = "_ZN2da15bwd_dkdv_kernelILi64ELi0ELb0ELb0EEEvN6da_abi10BwdParamsTIDF16_EE"
+    fwd_plain = "_ZN2da10fwd_kernelILi64ELb1ELi0ELb0EEEvN6da_abi10FwdParamsTIDF16_EE"
+    fwd_drop = "_ZN2da10fwd_kernelILi64ELb1ELi1ELb1EEEvN6da_abi10FwdParamsTIDF16_EE"
+    build.check_resources("x.hip", remark % (dkdv, 0) + remark % (fwd_plain, 0) + remark % (fwd_drop, 24))
+    for name in (dkdv, fwd_plain):
+        with pytest.raises(RuntimeError, match="must not spill"):
+            build.check_resources("x.hip", remark % (dkdv, 0) + remark % (name, 16))

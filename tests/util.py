@@ -1,20 +1,12 @@
 """Shared helpers of the parity tests: seeded synthetic inputs and the tolerance metrics."""
 import torch
 
+from synthetic import make_inputs  # noqa: F401  (the benchmark draws the same tensors)
+
 # tolerances stated by the build's target: outputs within max-abs 2e-2 of the fp32 oracle,
 # gradients within 5e-2 relative to the max-norm of the oracle gradient
 Y_ATOL = 2e-2
 GRAD_RTOL = 5e-2
-
-
-def make_inputs(B, H, N, D, seed, scale=1.0, with_dy=True):
-    """fp16 tensors drawn i.i.d. N(0, scale^2) on the CPU in the fixed order q1,q2,k1,k2,v,dy."""
-    g = torch.Generator().manual_seed(seed)
-    mk = lambda d: (torch.randn(B, H, N, d, generator=g, dtype=torch.float32) * scale).to(torch.float16)
-    q1, q2, k1, k2 = mk(D), mk(D), mk(D), mk(D)
-    v = mk(2 * D)
-    dy = (torch.randn(B, H, N, 2 * D, generator=g, dtype=torch.float32)).to(torch.float16) if with_dy else None
-    return q1, q2, k1, k2, v, dy
 
 
 def max_abs(a, b):

@@ -11,7 +11,7 @@ import torch  # noqa: F401  (must precede loading the library)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libdiffattn.so")
 
-ABI_VERSION = 6   # the version of include/diffattn.h this binding is written against
+ABI_VERSION = 7   # the version of include/diffattn.h this binding is written against
 
 _lib = None
 
@@ -20,9 +20,11 @@ _fp = ctypes.c_void_p  # float* passed as raw addresses
 
 
 class Layout(ctypes.Structure):
-    """diffattn_layout: element strides (batch, head, row) of q/k, v, y and dy."""
+    """diffattn_layout: element strides (batch, head, row) of q/k, v, y, dy and of the gradients of q/k and v
+    (gradient strides left at zero mean dense)."""
     _fields_ = [(n, ctypes.c_longlong) for n in (
-        "qk_b", "qk_h", "qk_n", "v_b", "v_h", "v_n", "y_b", "y_h", "y_n", "dy_b", "dy_h", "dy_n")]
+        "qk_b", "qk_h", "qk_n", "v_b", "v_h", "v_n", "y_b", "y_h", "y_n", "dy_b", "dy_h", "dy_n",
+        "dqk_b", "dqk_h", "dqk_n", "dv_b", "dv_h", "dv_n")]
 
 
 class Dropout(ctypes.Structure):

@@ -27,10 +27,15 @@ def _rms(x: torch.Tensor) -> torch.Tensor:
     return F.rms_norm(x, (x.size(-1),), eps=RMS_EPS)
 
 
-def _per_head(lambda_scale):
-    """A lambda tensor with one value per head broadcasts over [B, H, N, *]; one value or a number stays."""
-    if torch.is_tensor(lambda_scale) and lambda_scale.numel() > 1:
-        return lambda_scale.reshape(1, -1, 1, 1)
+def _per_head(lambda_scale, dtype=None):
+    """A lambda tensor with one value per head broadcasts over [B, H, N, *]; one value or a number stays.
+    A tensor is brought to the dtype of the probabilities it multiplies (an fp32 lambda would otherwise
+    promote them and then meet v in another dtype)."""
+    if torch.is_tensor(lambda_scale):
+        if dtype is not None:
+            lambda_scale = lambda_scale.to(dtype)
+        if lambda_scale.numel() > 1:
+            return lambda_scale.reshape(1, -1, 1, 1)
     return lambda_scale
 
 
@@ -50,7 +55,7 @@ def MultiheadAttn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, rms_norm: b
 
 def MultiheadDiffAttn(q1, q2, k1, k2, v, lambda_scale=-0.5, lambda_init: float = 0.8, rms_norm: bool = False,
                       causal: bool = False):
-    weights = _probabilities(q1, k1, causal) - _per_head(lambda_scale) * _probabilities(q2, k2, causal)
+    weights = _probabilities(q1, k1, causal) - _per_head(lambda_scale, q1.dtype) * _probabilities(q2, k2, causal)
     out = weights @ v
     if rms_norm:
         out = (1 - lambda_init) * _rms(out)
@@ -68,7 +73,7 @@ def MultiheadFlashDiffAttn(q1, q2, k1, k2, v, lambda_scale=-0.5, lambda_init: fl
     halves = v.split(q1.size(-1), dim=-1)
     stream1 = torch.cat([F.scaled_dot_product_attention(q1, k1, h, is_causal=causal) for h in halves], dim=-1)
     stream2 = torch.cat([F.scaled_dot_product_attention(q2, k2, h, is_causal=causal) for h in halves], dim=-1)
-    out = stream1 - _per_head(lambda_scale) * stream2
+    out = stream1 - _per_head(lambda_scale, q1.dtype) * stream2
     if rms_norm:
         out = (1 - lambda_init) * _rms(out)
     return out

@@ -20,6 +20,29 @@ FLAGS = [
     "-fno-honor-nans",
     "-Wno-unused-command-line-argument",
 ]
+# the kernel sources are compiled with per-kernel resource remarks, which check_resources() reads
+REMARKS = ["-Rpass-analysis=kernel-resource-usage"]
+
+
+def check_resources(src, remarks):
+    """Fails the build when a kernel that must not spill uses scratch memory.
+
+    The dK/dV kernels issue some of their matrix products as inline assembly, for which the compiler places no
+    wait states: a spilled operand reloaded (scratch_load, or v_accvgpr_write of a parked copy) directly in
+    front of such a product would be read too early, silently.  The register budgets are sized by hand so
+    that nothing spills; this holds the build to it.  Backward kernels: none may use scratch.  Forward
+    kernels: those without dropout (last template argument) may not.
+    """
+    import re
+    bad = []
+    for name, scratch in re.findall(r"Function Name: (\S+).*?ScratchSize \[bytes/lane\]: (\d+)", remarks, re.S):
+        if int(scratch) == 0:
+            continue
+        dropout = name.split("EEEv")[0].endswith("Lb1")
+        if "bwd_" in name or ("fwd_kernel" in name and not dropout):
+            bad.append("%s: %s bytes of scratch per lane" % (name, scratch))
+    if bad:
+        raise RuntimeError("%s: kernels that must not spill do:\n  %s" % (src, "\n  ".join(bad)))
 
 
 def build(verbose=True):
@@ -30,16 +53,20 @@ def build(verbose=True):
     units += [(src, ["-DDA_BF16"], src.replace(".hip", "_bf16.o")) for src in KERNEL_SOURCES]
     for src, extra, obj_name in units:
         obj = os.path.join(CSRC, obj_name)
-        cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+        remarks = REMARKS if src in KERNEL_SOURCES else []
+        cmd = [HIPCC, *FLAGS, *remarks, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
-        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        procs.append((src, cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs.append(obj)
-    for cmd, pr in procs:
+    for src, cmd, pr in procs:
         out, _ = pr.communicate()
-        out = "\n".join(l for l in out.splitlines() if "is not a recognized feature" not in l)
         if pr.returncode != 0:
+            out = "\n".join(l for l in out.splitlines() if "is not a recognized feature" not in l and "remark:" not in l)
             raise RuntimeError("hipcc failed: %s\n%s" % (" ".join(cmd), out))
+        if src in KERNEL_SOURCES:
+            check_resources(src, out)
+        out = "\n".join(l for l in out.splitlines() if "is not a recognized feature" not in l and "remark:" not in l)
         if verbose and out.strip():
             print(out)
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]

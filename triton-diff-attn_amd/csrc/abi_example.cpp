@@ -6,7 +6,8 @@
 //
 // With a third argument the tensors q1, q2, k1, k2, v, dy of in.bin and y of out.bin are stored
 // [B,N,H,C] (the layout a projection writes) and are handed to the library as they are, through the
-// strides of diffattn_layout; the gradients always come back dense [B,H,N,C].
+// strides of diffattn_layout; the gradient strides of the layout are left zero, so the gradients come
+// back dense [B,H,N,C].
 //
 // in.bin : int32 B, H, N, D, flags; float32 lambda_init, sm_scale; then the 16-bit tensors q1, q2, k1,
 //          k2 [B,H,N,D], v, dy [B,H,N,2D] and lambda (1 or H values), all in the dtype the flags name

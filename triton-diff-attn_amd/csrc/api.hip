@@ -23,7 +23,8 @@ hipError_t launch_bwd(const BwdParams& p, int D, hipStream_t stream);
 
 namespace {
 
-constexpr int kKnownFlags = DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL | DIFFATTN_BF16 | DIFFATTN_LAMBDA_PER_HEAD;
+constexpr int kKnownFlags = DIFFATTN_RMS_NORM | DIFFATTN_CAUSAL | DIFFATTN_BF16 | DIFFATTN_LAMBDA_PER_HEAD | DIFFATTN_LAMBDA_FP32 |
+                            DIFFATTN_UNPADDED;
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -58,8 +59,9 @@ int static_scratch(void** out) {
   return DIFFATTN_OK;
 }
 
-// Layout of the strided tensors: the caller's, or dense [B,H,N,C] when none is given.
-struct Layouts { da_abi::Strides qk, v, y, dy; };
+// Layout of the caller's tensors: the given strides, or dense [B,H,rows,C] where none are given; `rows` is
+// N, or n_valid with DIFFATTN_UNPADDED.
+struct Layouts { da_abi::Strides qk, v, y, dy, dqk, dv; };
 
 inline da_abi::Strides dense(int H, int N, int C) { return {(long long)H * N * C, (long long)N * C, (long long)C}; }
 
@@ -69,17 +71,32 @@ inline bool stride_ok(long long b, long long h, long long n, int C) {
   return n >= C && n % 8 == 0 && n <= (1LL << 26) && b >= 0 && h >= 0 && b % 8 == 0 && h % 8 == 0;
 }
 
-int resolve_layout(const diffattn_layout* l, int H, int N, int D, Layouts* out) {
-  out->qk = dense(H, N, D);
-  out->v = out->y = out->dy = dense(H, N, 2 * D);
+// a tensor that is written must not lie on top of itself (an input may be broadcast with a zero stride)
+inline bool no_overlap(long long b, long long h, int B, int H) { return (B == 1 || b != 0) && (H == 1 || h != 0); }
+
+// `backward`: the backward reads dy and writes the gradients through their strides; the forward ignores those
+// fields, so a caller of the forward may leave them zero.  Gradient strides that are all zero mean dense.
+int resolve_layout(const diffattn_layout* l, int B, int H, int rows, int D, bool backward, Layouts* out) {
+  out->qk = out->dqk = dense(H, rows, D);
+  out->v = out->y = out->dy = out->dv = dense(H, rows, 2 * D);
   if (!l) return DIFFATTN_OK;
   if (!stride_ok(l->qk_b, l->qk_h, l->qk_n, D) || !stride_ok(l->v_b, l->v_h, l->v_n, 2 * D) ||
-      !stride_ok(l->y_b, l->y_h, l->y_n, 2 * D) || !stride_ok(l->dy_b, l->dy_h, l->dy_n, 2 * D))
+      !stride_ok(l->y_b, l->y_h, l->y_n, 2 * D))
     return DIFFATTN_EINVAL_LAYOUT;
   out->qk = {l->qk_b, l->qk_h, l->qk_n};
   out->v = {l->v_b, l->v_h, l->v_n};
   out->y = {l->y_b, l->y_h, l->y_n};
+  if (!backward) return no_overlap(l->y_b, l->y_h, B, H) ? DIFFATTN_OK : DIFFATTN_EINVAL_LAYOUT;
+  if (!stride_ok(l->dy_b, l->dy_h, l->dy_n, 2 * D)) return DIFFATTN_EINVAL_LAYOUT;
   out->dy = {l->dy_b, l->dy_h, l->dy_n};
+  if (l->dqk_b || l->dqk_h || l->dqk_n) {
+    if (!stride_ok(l->dqk_b, l->dqk_h, l->dqk_n, D) || !no_overlap(l->dqk_b, l->dqk_h, B, H)) return DIFFATTN_EINVAL_LAYOUT;
+    out->dqk = {l->dqk_b, l->dqk_h, l->dqk_n};
+  }
+  if (l->dv_b || l->dv_h || l->dv_n) {
+    if (!stride_ok(l->dv_b, l->dv_h, l->dv_n, 2 * D) || !no_overlap(l->dv_b, l->dv_h, B, H)) return DIFFATTN_EINVAL_LAYOUT;
+    out->dv = {l->dv_b, l->dv_h, l->dv_n};
+  }
   return DIFFATTN_OK;
 }
 
@@ -107,7 +124,7 @@ __global__ __launch_bounds__(256) void dropout_mask_kernel(unsigned char* keep, 
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (size_t)N * N) return;
   const unsigned q = (unsigned)(idx / N), k = (unsigned)(idx % N);
-  const unsigned word = dropout_word(cfg, 2u * bh + stream, (unsigned)N / 2, q >> 1, k >> 1);
+  const unsigned word = dropout_word(dropout_key(cfg, 2u * bh + stream), (unsigned)N / 2, q >> 1, k >> 1);
   keep[(size_t)bh * N * N + idx] = dropout_keep(word, q, k, cfg.threshold) ? 1 : 0;
 }
 
@@ -143,6 +160,7 @@ void fill_fwd(da_abi::FwdParamsT<T>& p, const void* q1, const void* q2, const vo
   p.causal = (flags & DIFFATTN_CAUSAL) ? 1 : 0;
   p.n_keys = n_valid;
   p.H = H; p.lambda_stride = (flags & DIFFATTN_LAMBDA_PER_HEAD) ? 1 : 0;
+  p.lambda_fp32 = (flags & DIFFATTN_LAMBDA_FP32) ? 1 : 0;
 }
 
 template <class T>
@@ -154,7 +172,7 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
               int BH, int H, int N, int n_valid, float sm_scale, float lambda_init, int flags, unsigned stage_mask,
               const Layouts& lay, const da_abi::DropoutCfg& drop) {
   p.drop = drop;
-  p.sqk = lay.qk; p.sv = lay.v; p.sy = lay.y; p.sdy = lay.dy;
+  p.sqk = lay.qk; p.sv = lay.v; p.sy = lay.y; p.sdy = lay.dy; p.sdqk = lay.dqk; p.sdv = lay.dv;
   p.q1 = (const T*)q1; p.q2 = (const T*)q2; p.k1 = (const T*)k1; p.k2 = (const T*)k2;
   p.v = (const T*)v; p.lambda_scale = (const T*)lambda_scale;
   p.y = (const T*)y; p.u2 = (const T*)u2; p.lse1 = lse1; p.lse2 = lse2; p.rinv = rinv;
@@ -168,13 +186,14 @@ void fill_bwd(da_abi::BwdParamsT<T>& p, const void* q1, const void* q2, const vo
   p.n_keys = n_valid;
   p.stages = stage_mask & DIFFATTN_STAGE_ALL;
   p.H = H; p.lambda_stride = (flags & DIFFATTN_LAMBDA_PER_HEAD) ? 1 : 0;
+  p.lambda_fp32 = (flags & DIFFATTN_LAMBDA_FP32) ? 1 : 0;
 }
 
 }  // namespace
 
 extern "C" {
 
-int diffattn_abi_version(void) { return 6; }
+int diffattn_abi_version(void) { return 7; }
 
 const char* diffattn_strerror(int code) {
   switch (code) {
@@ -185,9 +204,9 @@ const char* diffattn_strerror(int code) {
     case DIFFATTN_EINVAL_WS: return "workspace too small or misaligned";
     case DIFFATTN_EINVAL_ALIGN: return "tensor pointers must be 16-byte aligned";
     case DIFFATTN_EINVAL_SCRATCH: return "problem too large for the built-in scratch of diffattn_backward_static (DIFFATTN_STATIC_SCRATCH_BYTES): use diffattn_backward with a caller workspace";
-    case DIFFATTN_EINVAL_LAYOUT: return "bad strides in diffattn_layout: every stride must be a non-negative multiple of 8 elements and a row stride at least the row width";
+    case DIFFATTN_EINVAL_LAYOUT: return "bad strides in diffattn_layout: every stride must be a non-negative multiple of 8 elements, a row stride at least the row width, and the batch and head strides of a tensor that is written non-zero";
     case DIFFATTN_EINVAL_DROPOUT: return "dropout probability must lie in [0, 255/256]";
-    case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL, DIFFATTN_BF16, DIFFATTN_LAMBDA_PER_HEAD)";
+    case DIFFATTN_EINVAL_FLAGS: return "unknown bits in flags (known: DIFFATTN_RMS_NORM, DIFFATTN_CAUSAL, DIFFATTN_BF16, DIFFATTN_LAMBDA_PER_HEAD, DIFFATTN_LAMBDA_FP32, DIFFATTN_UNPADDED)";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -214,7 +233,7 @@ int diffattn_forward_padded(const void* q1, const void* q2, const void* k1, cons
       !aligned16(y) || !aligned16(u2))
     return DIFFATTN_EINVAL_ALIGN;
   Layouts lay;
-  if (int e = resolve_layout(layout, H, N, D, &lay)) return e;
+  if (int e = resolve_layout(layout, B, H, (flags & DIFFATTN_UNPADDED) ? n_valid : N, D, false, &lay)) return e;
   da_abi::DropoutCfg drop;
   if (int e = resolve_dropout(dropout, &drop)) return e;
   if (flags & DIFFATTN_BF16) {
@@ -254,7 +273,7 @@ int diffattn_backward_stages(const void* q1, const void* q2, const void* k1, con
   for (const void* q : ptrs)
     if (!aligned16(q)) return DIFFATTN_EINVAL_ALIGN;
   Layouts lay;
-  if (int e = resolve_layout(layout, H, N, D, &lay)) return e;
+  if (int e = resolve_layout(layout, B, H, (flags & DIFFATTN_UNPADDED) ? n_valid : N, D, true, &lay)) return e;
   da_abi::DropoutCfg drop;
   if (int e = resolve_dropout(dropout, &drop)) return e;
   const WsLayout w = ws_layout(B * H, N, D);

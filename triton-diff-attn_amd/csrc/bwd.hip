@@ -45,9 +45,17 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
     const size_t row = (size_t)blockIdx.x * kPrepRows + pass * RPP + rloc;
     const size_t off = row * DV + 8 * sub;
     const size_t n = (size_t)(n0 + pass * RPP + rloc);
-    const h8 y8 = *reinterpret_cast<const h8*>(gy + n * (size_t)p.sy.n);
+    // a padding row (past the sequence's real length) has no y and dy rows: it gets dX = 0 and zero statistics,
+    // so it adds nothing to dK, dV and d(lambda)
+    const bool real = n < (size_t)p.n_keys;
+    h8 y8, g8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { y8[e] = (half_t)0.f; g8[e] = (half_t)0.f; }
+    if (real) {
+      y8 = *reinterpret_cast<const h8*>(gy + n * (size_t)p.sy.n);
+      g8 = *reinterpret_cast<const h8*>(gdy + n * (size_t)p.sdy.n);
+    }
     const h8 u8 = *reinterpret_cast<const h8*>(p.u2 + off);
-    const h8 g8 = *reinterpret_cast<const h8*>(gdy + n * (size_t)p.sdy.n);
     float dx[8], x[8];
     if (RMS) {
       float gy = 0.f;
@@ -110,7 +118,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
 // consecutive partials belong to a unit.  One workgroup per output; its first 256 threads add in a fixed
 // order whatever the size of the workgroup, so the result does not depend on the kernel that hosts it.
 __device__ __forceinline__ void dlambda_reduce(const float* __restrict__ part, int per_unit, int n_units, half_t* out,
-                                               int o, int n_out, float* red) {
+                                               int o, int n_out, float* red, int out_fp32) {
   const int tid = threadIdx.x;
   const int n = (n_units / n_out) * per_unit;        // partials this workgroup sums
   float acc = 0.f;
@@ -128,13 +136,18 @@ __device__ __forceinline__ void dlambda_reduce(const float* __restrict__ part, i
     if (tid < s) red[tid] += red[tid + s];
     __syncthreads();
   }
-  if (tid == 0) out[o] = (half_t)red[0];
+  if (tid == 0) {
+    // the sum leaves the library in the 16-bit type of the tensors, like the reference's (src/kernel.py:573),
+    // or unrounded in fp32 when the caller keeps lambda in fp32
+    if (out_fp32) reinterpret_cast<float*>(out)[o] = red[0];
+    else out[o] = (half_t)red[0];
+  }
 }
 
 __global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restrict__ part, int per_unit, int n_units,
-                                                          half_t* out) {
+                                                          half_t* out, int out_fp32) {
   __shared__ float red[256];
-  dlambda_reduce(part, per_unit, n_units, out, blockIdx.x, gridDim.x, red);
+  dlambda_reduce(part, per_unit, n_units, out, blockIdx.x, gridDim.x, red, out_fp32);
 }
 
 // The dK/dV and dQ kernels can host that reduction in p.dlam_fold extra workgroups at the end of their grid
@@ -142,7 +155,7 @@ __global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restric
 #define DA_HOST_DLAMBDA(smem_)                                                                                  \
   if (p.dlam_fold && (int)blockIdx.x >= (int)gridDim.x - p.dlam_fold) {                                         \
     dlambda_reduce(p.dlam_part, p.n_part / p.BH, p.BH, p.dlambda, (int)blockIdx.x - ((int)gridDim.x - p.dlam_fold), \
-                   p.dlam_fold, reinterpret_cast<float*>(smem_));                                               \
+                   p.dlam_fold, reinterpret_cast<float*>(smem_), p.lambda_fp32);                                \
     return;                                                                                                     \
   }
 
@@ -181,7 +194,10 @@ struct DkvCfg {
 // DROP: dropout on both softmax maps, masks regenerated from the hash the forward used.  With the
 // keep mask m_t and c = 1/(1-p):  dS1 = A1 (c m1 dP - delta1),  dS2 = A2 (-lambda c m2 dP - delta2),
 // dV = c (m1 A1 - lambda m2 A2)^T dX; delta1, delta2 are the row dots with the dropped-out U1, U2.
-template <int D, int MODE, bool CAUSAL, bool DROP>
+// PADDED: rows n_keys..N-1 are padding.  As queries they read the last real row of Q1 and Q2 (the row the
+// forward used for their logsumexp) and carry dX = 0; as keys they read the last real row of K1, K2, V and
+// their results are not stored.
+template <int D, int MODE, bool CAUSAL, bool DROP, bool PADDED>
 __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_kernel(BwdParams p) {
   using C = DkvCfg<D>;
   constexpr int DV = C::DV, NW = C::NW, BK = C::BK, BQ = C::BQ;
@@ -208,19 +224,22 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   const size_t rows = (size_t)p.BH * p.N;
   const size_t row0 = (size_t)bh * p.N;
   const int key = kt * BK + wave * 32 + j;
+  const int key_row = (PADDED && key >= p.n_keys) ? p.n_keys - 1 : key;    // the row this lane's key is read from
   // element offsets of the unit's first row and the row strides of the strided tensors
   const size_t qk_base = da_abi::unit_base(p, p.sqk, bh), v_base = da_abi::unit_base(p, p.sv, bh);
   const int qk_n = (int)p.sqk.n, v_n = (int)p.sv.n;
 
   const float c = p.sm_scale * kLog2e;
   const float lam = da_abi::lambda_of_unit(p, bh);
+  // hash keys of this unit's two softmax streams (used with dropout only)
+  const DropoutKey dkey1 = dropout_key(p.drop, 2u * bh), dkey2 = dropout_key(p.drop, 2u * bh + 1);
 
   // persistent B operands: this lane's key row of K1, K2, V
   h8 kf1[NKS], kf2[NKS], vf[NKV];
   {
-    const half_t* r1 = p.k1 + qk_base + (size_t)key * qk_n + 8 * g;
-    const half_t* r2 = p.k2 + qk_base + (size_t)key * qk_n + 8 * g;
-    const half_t* rv = p.v + v_base + (size_t)key * v_n + 8 * g;
+    const half_t* r1 = p.k1 + qk_base + (size_t)key_row * qk_n + 8 * g;
+    const half_t* r2 = p.k2 + qk_base + (size_t)key_row * qk_n + 8 * g;
+    const half_t* rv = p.v + v_base + (size_t)key_row * v_n + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       // pre-multiplied by sm_scale*log2(e): the score products come out in log2 units
@@ -267,11 +286,15 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   auto stage = [&](int qt, int buf, int part) {
     half_t* bq = smem + buf * (C::QBUF / 2);
     half_t* bx = smem + (C::XBASE + buf * C::XBUF) / 2;
+    // dX and the statistics come from the workspace, which has all N rows; Q1 and Q2 have n_keys
+    const bool past_end = PADDED && (qt + 1) * BQ > p.n_keys;
     if (part == 0) {
-      QTile::issue_at(gq1 + (size_t)qt * BQ * qk_n, bq, wave, lane, q_off, qk_n);
+      if (past_end) QTile::issue_clamped(gq1 + (size_t)qt * BQ * qk_n, bq, wave, lane, q_off, qk_n, p.n_keys - 1 - qt * BQ);
+      else QTile::issue_at(gq1 + (size_t)qt * BQ * qk_n, bq, wave, lane, q_off, qk_n);
       if (wave == 0 && lane < BQ) async_copy16(reinterpret_cast<const half_t*>(gstat + (size_t)qt * BQ), stat_off, smem + (C::SBASE + buf * C::SBUF) / 2);
     } else if (part == 1) {
-      QTile::issue_at(gq2 + (size_t)qt * BQ * qk_n, bq + C::Q_TILE, wave, lane, q_off, qk_n);
+      if (past_end) QTile::issue_clamped(gq2 + (size_t)qt * BQ * qk_n, bq + C::Q_TILE, wave, lane, q_off, qk_n, p.n_keys - 1 - qt * BQ);
+      else QTile::issue_at(gq2 + (size_t)qt * BQ * qk_n, bq + C::Q_TILE, wave, lane, q_off, qk_n);
     } else if (part == 2) {
       XTile::template issue<0, XH>(gx + (size_t)qt * BQ * DV, bx, wave, lane);
     } else {
@@ -392,8 +415,8 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
       // share the hash words of their 2x2 block, one word per softmax stream
       const unsigned query = (unsigned)(qbase + 8 * (r / 4) + (r % 4));
       if ((r & 1) == 0) {
-        t.w1 = dropout_word(p.drop, 2u * bh, (unsigned)p.N / 2, query >> 1, (unsigned)key >> 1);
-        t.w2 = dropout_word(p.drop, 2u * bh + 1, (unsigned)p.N / 2, query >> 1, (unsigned)key >> 1);
+        t.w1 = dropout_word(dkey1, (unsigned)p.N / 2, query >> 1, (unsigned)key >> 1);
+        t.w2 = dropout_word(dkey2, (unsigned)p.N / 2, query >> 1, (unsigned)key >> 1);
       }
       const bool keep1 = dropout_keep(t.w1, query, (unsigned)key, p.drop.threshold);
       const bool keep2 = dropout_keep(t.w2, query, (unsigned)key, p.drop.threshold);
@@ -635,24 +658,28 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
 
   wait_async_tiles();   // the re-fetch issued by the last step has nothing left to land in after the kernel
   // accumulator tile tt: column = 32*tt + j (feature), register r = key row 8*(r/4) + 4g + (r%4)
-  const size_t krow0 = row0 + (size_t)kt * BK + wave * 32;
+  const int kloc0 = kt * BK + wave * 32;               // first key of this wave inside the unit
   if constexpr (DO_V) {
+    half_t* const o = p.dv + da_abi::unit_base(p, p.sdv, bh) + (size_t)kloc0 * (size_t)p.sdv.n;
 #pragma unroll
     for (int tt = 0; tt < NVT; ++tt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int kr = 8 * (r / 4) + 4 * g + (r % 4);
-        p.dv[(krow0 + kr) * DV + 32 * tt + j] = (half_t)dv[tt][r];
+        if (!PADDED || kloc0 + kr < p.n_keys) o[(size_t)kr * (size_t)p.sdv.n + 32 * tt + j] = (half_t)dv[tt][r];
       }
   }
   if constexpr (DO_K) {
+    const size_t ob = da_abi::unit_base(p, p.sdqk, bh) + (size_t)kloc0 * (size_t)p.sdqk.n;
 #pragma unroll
     for (int tt = 0; tt < NDT; ++tt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int kr = 8 * (r / 4) + 4 * g + (r % 4);
-        p.dk1[(krow0 + kr) * D + 32 * tt + j] = (half_t)(dk1[tt][r] * p.sm_scale);
-        p.dk2[(krow0 + kr) * D + 32 * tt + j] = (half_t)(dk2[tt][r] * p.sm_scale);
+        if (!PADDED || kloc0 + kr < p.n_keys) {
+          p.dk1[ob + (size_t)kr * (size_t)p.sdqk.n + 32 * tt + j] = (half_t)(dk1[tt][r] * p.sm_scale);
+          p.dk2[ob + (size_t)kr * (size_t)p.sdqk.n + 32 * tt + j] = (half_t)(dk2[tt][r] * p.sm_scale);
+        }
       }
   }
 }
@@ -688,6 +715,9 @@ template <int D, int NWAVES, int MASK, bool DROP>
 __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_waves_per_eu(DqCfg<D, NWAVES>::OCC, DqCfg<D, NWAVES>::OCC))) void bwd_dq_kernel(BwdParams p) {
   using C = DqCfg<D, NWAVES>;
   constexpr bool CAUSAL = (MASK == 1), PADDED = (MASK == 2);
+  // rows past the real length are neither read from the caller's tensors nor written to the gradients: checked
+  // in both masked variants (the causal one serves padded sequences too), compiled out of the plain one
+  constexpr bool TAIL = (MASK != 0);
   constexpr int DV = C::DV, NW = C::NW, BM = C::BM, BN = C::BN;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
 
@@ -716,6 +746,8 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   const int qk_n = (int)p.sqk.n, v_n = (int)p.sv.n;
 
   const float lam = da_abi::lambda_of_unit(p, bh);
+  // hash keys of this unit's two softmax streams (used with dropout only)
+  const DropoutKey dkey1 = dropout_key(p.drop, 2u * bh), dkey2 = dropout_key(p.drop, 2u * bh + 1);
 
   // persistent B operands: this lane's query row of Q1, Q2 (pre-multiplied by sm_scale*log2(e)
   // exactly as in the forward kernel, so the recomputed probabilities match it), dX, and its row
@@ -723,8 +755,11 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   h8 qf1[NKS], qf2[NKS], xf[NKV];
   {
     const float c = p.sm_scale * kLog2e;
-    const half_t* r1 = p.q1 + qk_base + (size_t)(qt * BM + wave * 32 + j) * qk_n + 8 * g;
-    const half_t* r2 = p.q2 + qk_base + (size_t)(qt * BM + wave * 32 + j) * qk_n + 8 * g;
+    // a padding row stands in with the last real row, as in the forward; its results are not stored
+    int qr = qt * BM + wave * 32 + j;
+    if (TAIL && qr >= p.n_keys) qr = p.n_keys - 1;
+    const half_t* r1 = p.q1 + qk_base + (size_t)qr * qk_n + 8 * g;
+    const half_t* r2 = p.q2 + qk_base + (size_t)qr * qk_n + 8 * g;
     const half_t* rx = p.dx + qrow * DV + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
@@ -758,11 +793,24 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   constexpr int VH = (VTile::PER + 1) / 2;
 
   const int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
+  // with padding, the tiles that reach past the last real key are copied with their row index clamped to it
+  auto copy_k = [&](const half_t* gk, int t, half_t* dst) {
+    if (TAIL && (t + 1) * BN > p.n_keys) KTile::issue_clamped(gk + (size_t)t * BN * qk_n, dst, wave, lane, k_off, qk_n, p.n_keys - 1 - t * BN);
+    else KTile::issue_at(gk + (size_t)t * BN * qk_n, dst, wave, lane, k_off, qk_n);
+  };
+  auto copy_v = [&](int t, half_t* dst, auto k0_tag, auto k1_tag) {
+    constexpr int K0 = decltype(k0_tag)::value, K1 = decltype(k1_tag)::value;
+    if (TAIL && (t + 1) * BN > p.n_keys) VTile::template issue_clamped<K0, K1>(gv + (size_t)t * BN * v_n, dst, wave, lane, v_off, v_n, p.n_keys - 1 - t * BN);
+    else VTile::template issue_at<K0, K1>(gv + (size_t)t * BN * v_n, dst, wave, lane, v_off, v_n);
+  };
+  constexpr std::integral_constant<int, 0> v_begin{};
+  constexpr std::integral_constant<int, VH> v_mid{};
+  constexpr std::integral_constant<int, VTile::PER> v_end{};
   auto fetch_all = [&](int t, int buf) {
     half_t* b = smem + buf * C::STAGE;
-    KTile::issue_at(gk1 + (size_t)t * BN * qk_n, b, wave, lane, k_off, qk_n);
-    KTile::issue_at(gk2 + (size_t)t * BN * qk_n, b + C::K_TILE, wave, lane, k_off, qk_n);
-    VTile::issue_at(gv + (size_t)t * BN * v_n, b + 2 * C::K_TILE, wave, lane, v_off, v_n);
+    copy_k(gk1, t, b);
+    copy_k(gk2, t, b + C::K_TILE);
+    copy_v(t, b + 2 * C::K_TILE, v_begin, v_end);
   };
   fetch_all(0, 0);
   fetch_all((n_tiles > 1) ? 1 : 0, 1);
@@ -779,11 +827,11 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
     const half_t* sV = sK1 + 2 * C::K_TILE;
     half_t* nb = smem + bnext * C::STAGE;            // held tile t-1, consumed one iteration ago
     const int tn = (t + 2 < n_tiles) ? t + 2 : n_tiles - 1;   // past the end: harmless re-reads
-    KTile::issue_at(gk1 + (size_t)tn * BN * qk_n, nb, wave, lane, k_off, qk_n);
+    copy_k(gk1, tn, nb);
 
 #pragma unroll
     for (int ksub = 0; ksub < BN / 32; ++ksub) {
-      if (ksub == 0) KTile::issue_at(gk2 + (size_t)tn * BN * qk_n, nb + C::K_TILE, wave, lane, k_off, qk_n);
+      if (ksub == 0) copy_k(gk2, tn, nb + C::K_TILE);
       // transposed tiles [32 keys x 32 queries]: this lane's column is its query
       f16v s1, s2, dp;
 #pragma unroll
@@ -806,8 +854,8 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       }
 #pragma unroll
       for (int kv = 0; kv < NKV; ++kv) dp = mfma32(av[kv], xf[kv], dp);
-      if (ksub == 0) VTile::template issue_at<0, VH>(gv + (size_t)tn * BN * v_n, nb + 2 * C::K_TILE, wave, lane, v_off, v_n);
-      if (ksub == BN / 32 - 1) VTile::template issue_at<VH, VTile::PER>(gv + (size_t)tn * BN * v_n, nb + 2 * C::K_TILE, wave, lane, v_off, v_n);
+      if (ksub == 0) copy_v(tn, nb + 2 * C::K_TILE, v_begin, v_mid);
+      if (ksub == BN / 32 - 1) copy_v(tn, nb + 2 * C::K_TILE, v_mid, v_end);
       if constexpr (CAUSAL) {
         // only the last sub-tiles of a wave's loop reach past its first row: mask key > query there
         const int wrow0 = qt * BM + wave * 32;
@@ -842,7 +890,10 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
         tk2[kk][tt] = join(lds_read_tr(sK2 + swz_off<D>(rbase, 32 * tt + tr_col)),
                            lds_read_tr(sK2 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
       };
-      if constexpr (!DROP) {
+      // (At D = 128 the masked variants, which also carry the row clamping of padded sequences, are short of
+      // registers in the same way.)
+      constexpr bool kFragmentsAhead = !DROP && !(D == 128 && TAIL);
+      if constexpr (kFragmentsAhead) {
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
@@ -861,8 +912,8 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
           const unsigned query = (unsigned)(qt * BM + wave * 32 + j);
           const unsigned kq = (unsigned)(t * BN + ksub * 32 + 4 * g + 8 * (r / 4) + (r % 4));
           if ((r & 1) == 0) {
-            w1 = dropout_word(p.drop, 2u * bh, (unsigned)p.N / 2, query >> 1, kq >> 1);
-            w2 = dropout_word(p.drop, 2u * bh + 1, (unsigned)p.N / 2, query >> 1, kq >> 1);
+            w1 = dropout_word(dkey1, (unsigned)p.N / 2, query >> 1, kq >> 1);
+            w2 = dropout_word(dkey2, (unsigned)p.N / 2, query >> 1, kq >> 1);
           }
           const float dpk = p.drop.keep_scale * dp[r];
           const float d1 = dropout_keep(w1, query, kq, p.drop.threshold) ? dpk : 0.f;
@@ -881,7 +932,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
         for (int tt = 0; tt < NDT; ++tt) {
-          if constexpr (DROP) read_tk(kk, tt);
+          if constexpr (!kFragmentsAhead) read_tk(kk, tt);
           dq1[tt] = mfma32(tk1[kk][tt], b1[kk], dq1[tt]);
           dq2[tt] = mfma32(tk2[kk][tt], b2[kk], dq2[tt]);
         }
@@ -920,15 +971,19 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   __builtin_amdgcn_wave_barrier();   // the rows are read back by other lanes of this wave only
   constexpr int LPR = D / 8;         // lanes per row
   constexpr int RPI = 64 / LPR;      // rows per instruction
-  half_t* const o1 = p.dq1 + (row0 + qt * BM + wave * 32) * D;
-  half_t* const o2 = p.dq2 + (row0 + qt * BM + wave * 32) * D;
+  const int qloc0 = qt * BM + wave * 32;             // first query of this wave inside the unit
+  const size_t ob = da_abi::unit_base(p, p.sdqk, bh) + (size_t)qloc0 * (size_t)p.sdqk.n;
+  half_t* const o1 = p.dq1 + ob;
+  half_t* const o2 = p.dq2 + ob;
 #pragma unroll
   for (int k = 0; k < 32 / RPI; ++k) {
     const int row = k * RPI + lane / LPR, ch = lane % LPR;
     const u32x4 v1 = *reinterpret_cast<const u32x4*>(stg + row * SROW + 8 * ch);
     const u32x4 v2 = *reinterpret_cast<const u32x4*>(stg + (32 + row) * SROW + 8 * ch);
-    *reinterpret_cast<u32x4*>(o1 + (size_t)row * D + 8 * ch) = v1;
-    *reinterpret_cast<u32x4*>(o2 + (size_t)row * D + 8 * ch) = v2;
+    if (!TAIL || qloc0 + row < p.n_keys) {    // the gradient tensors have no rows past the real length
+      *reinterpret_cast<u32x4*>(o1 + (size_t)row * (size_t)p.sdqk.n + 8 * ch) = v1;
+      *reinterpret_cast<u32x4*>(o2 + (size_t)row * (size_t)p.sdqk.n + 8 * ch) = v2;
+    }
   }
 }
 
@@ -951,7 +1006,7 @@ static hipError_t launch_bwd_t(const BwdParams& p_in, hipStream_t stream) {
   }
   if ((p.stages & 2u) && !fold) {
     hipLaunchKernelGGL(bwd_dlambda_kernel, dim3(n_lambda), dim3(256), 0, stream,
-                       p.dlam_part, n_prep / p.BH, p.BH, p.dlambda);
+                       p.dlam_part, n_prep / p.BH, p.BH, p.dlambda, p.lambda_fp32);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
   if (p.stages & 4u) {
@@ -961,13 +1016,18 @@ static hipError_t launch_bwd_t(const BwdParams& p_in, hipStream_t stream) {
       p.dlam_fold = fold ? n_lambda : 0;
       fold = false;
       const dim3 grid(p.BH * (p.N / DkvCfg<D>::BK) + p.dlam_fold);
-      if (p.drop.threshold) {
-        if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, true, true>), grid, block, 0, stream, p);
-        else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, false, true>), grid, block, 0, stream, p);
-      } else {
-        if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, true, false>), grid, block, 0, stream, p);
-        else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, false, false>), grid, block, 0, stream, p);
-      }
+      auto launch_padded = [&](auto padded_tag) {
+        constexpr bool PAD = decltype(padded_tag)::value;
+        if (p.drop.threshold) {
+          if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, true, true, PAD>), grid, block, 0, stream, p);
+          else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, false, true, PAD>), grid, block, 0, stream, p);
+        } else {
+          if (p.causal) hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, true, false, PAD>), grid, block, 0, stream, p);
+          else          hipLaunchKernelGGL((bwd_dkdv_kernel<D, M, false, false, PAD>), grid, block, 0, stream, p);
+        }
+      };
+      if (p.n_keys < p.N) launch_padded(std::true_type{});
+      else                launch_padded(std::false_type{});
     };
     if constexpr (D == 128) {
       launch_mode(std::integral_constant<int, 1>{});

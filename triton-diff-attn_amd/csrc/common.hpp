@@ -236,6 +236,27 @@ struct AsyncTile {
   __device__ static __forceinline__ void issue(const half_t* gtile, half_t* lds_tile, int wave, int lane, int stride = COLS) {
     issue_at<K0, K1>(gtile, lds_tile, wave, lane, lane_off(wave, lane, stride), stride);
   }
+  // The same copy for a tile whose global rows end at `last_row` (relative to the tile's first row; it may be
+  // negative when the whole tile lies past the end): a row beyond it reads row `last_row` instead, so no
+  // address past the tensor's last row is formed and the LDS tile holds finite data everywhere.  Used for the
+  // last tiles of a sequence whose length is not a multiple of the tile; costs a few VALU instructions per piece.
+  template <int K0 = 0, int K1 = PER>
+  __device__ static __forceinline__ void issue_clamped(const half_t* gtile, half_t* lds_tile, int wave, int lane, unsigned off0,
+                                                       int stride, int last_row) {
+    const int r_l = lane / CPR;                        // the lane's row inside a piece
+#pragma unroll
+    for (int k = K0; k < K1; ++k) {
+      const int inst = wave + NW * k;
+      if (NINST % NW == 0 || inst < NINST) {
+        const int first = inst * RPP;                                  // first row of the piece
+        const int base_row = first < last_row ? first : last_row;     // wave-uniform
+        const int room = last_row - base_row;                          // rows the piece may advance: >= 0
+        const int back = r_l > room ? r_l - room : 0;                  // rows this lane steps back
+        const unsigned off = (kOneOffset ? off0 : lane_off(inst, lane, stride)) - (unsigned)(back * stride * 2);
+        async_copy16(gtile + (long long)base_row * stride, off, lds_tile + inst * 512);
+      }
+    }
+  }
 };
 
 __device__ __forceinline__ void wait_async_tiles() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
@@ -261,13 +282,34 @@ __device__ __forceinline__ void wait_async_tiles_except(int newest) {
 // mask dump agree without storing anything: one 32-bit word per 2x2 block of (query, key) pairs,
 // keyed on (seed, softmax stream, batch*head unit, query/2, key/2); the pair (q, k) owns byte
 // 2*(q&1) + (k&1) of the word and is kept iff that byte >= threshold, threshold = round(256 p).
+// The seed and the unit do not meet the counter directly: they are first mixed into two key words
+// (once per workgroup and stream), and the counter is hashed under both, one entering by XOR before the
+// first multiplication and one by addition after it.  Two seeds, however close, therefore give masks
+// that are not index permutations of each other.
 using da_abi::DropoutCfg;
 
-__device__ __forceinline__ unsigned dropout_word(const DropoutCfg& c, unsigned stream_unit, unsigned half_n, unsigned qh, unsigned kh) {
-  unsigned h = (qh * half_n + kh) ^ c.seed_lo;
+struct DropoutKey { unsigned k1, k2; };
+
+__device__ __forceinline__ DropoutKey dropout_key(const DropoutCfg& c, unsigned stream_unit) {
+  unsigned a = c.seed_lo ^ 0x9E3779B9u;
+  a *= 0x85EBCA6Bu; a ^= a >> 13;
+  a += c.seed_hi;
+  a *= 0xC2B2AE35u; a ^= a >> 16;
+  a += stream_unit;
+  a *= 0x27D4EB2Fu; a ^= a >> 15;
+  a *= 0x165667B1u; a ^= a >> 13;
+  unsigned b = a ^ 0x68E31DA4u;
+  b *= 0xB5297A4Du; b ^= b >> 15;
+  b += c.seed_hi ^ (stream_unit * 0x9E3779B1u);
+  b *= 0x1B56C4E9u; b ^= b >> 16;
+  return {a, b};
+}
+
+__device__ __forceinline__ unsigned dropout_word(const DropoutKey& key, unsigned half_n, unsigned qh, unsigned kh) {
+  unsigned h = (qh * half_n + kh) ^ key.k1;
   h *= 0x9E3779B1u;
   h ^= h >> 15;
-  h += (stream_unit * 0x85EBCA77u) ^ c.seed_hi;
+  h += key.k2;
   h *= 0xC2B2AE3Du;
   h ^= h >> 13;
   h *= 0x27D4EB2Fu;

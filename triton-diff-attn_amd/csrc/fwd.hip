@@ -71,6 +71,9 @@ void fwd_kernel(FwdParams p) {
 
   const int n_qt = p.N / BM;
   constexpr bool CAUSAL = (MASK == 1), PADDED = (MASK == 2);
+  // rows past the real length are neither read from the caller's tensors nor written to y: checked in both
+  // masked variants (the causal one serves padded sequences too), compiled out of the plain one
+  constexpr bool TAIL = (MASK != 0);
   int bh, qt;
   if constexpr (CAUSAL) {   // the last query block of a unit sees the most keys
     const UnitBlock ub = longest_first(blockIdx.x, p.BH);
@@ -84,6 +87,7 @@ void fwd_kernel(FwdParams p) {
   const size_t v_base = da_abi::unit_base(p, p.sv, bh);
   const int qk_n = (int)p.sqk.n, v_n = (int)p.sv.n;
   const int qrow0 = qt * BM + qw * 32 * QS + j;   // this lane's query row of block qs is qrow0 + 32*qs
+  const DropoutKey dkey = dropout_key(p.drop, 2u * bh + st);   // hash key of this wave's softmax stream (used with dropout only)
 
   // Q fragments (B operand): column j = this lane's query, k = 8g..8g+7 of each 16-wide k-step.
   // They are pre-multiplied by sm_scale*log2(e), so the MFMA result is the score in log2 units.
@@ -92,7 +96,11 @@ void fwd_kernel(FwdParams p) {
     const float c = p.sm_scale * kLog2e;
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
-      const half_t* r = (st ? p.q2 : p.q1) + qk_base + (size_t)(qrow0 + 32 * qs) * qk_n + 8 * g;
+      // a padding row (past the sequence's real length) stands in with the last real row: finite scores,
+      // results that are never stored
+      int qr = qrow0 + 32 * qs;
+      if (TAIL && qr >= p.n_keys) qr = p.n_keys - 1;
+      const half_t* r = (st ? p.q2 : p.q1) + qk_base + (size_t)qr * qk_n + 8 * g;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         h8 q = *reinterpret_cast<const h8*>(r + 16 * ks);
@@ -132,10 +140,31 @@ void fwd_kernel(FwdParams p) {
   static_assert(BM % (2 * BN) == 0, "an even number of key tiles per query block");
   constexpr int VH = (VTile::PER + 1) / 2;   // V instructions are issued in two groups
   const unsigned k_off = KTile::lane_off(wave, lane, qk_n), v_off = VTile::lane_off(wave, lane, v_n);
-  auto load_k1 = [&](int tk, int buf) { KTile::issue_at(gk1 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF, wave, lane, k_off, qk_n); };
-  auto load_k2 = [&](int tk, int buf) { KTile::issue_at(gk2 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF + C::K_TILE, wave, lane, k_off, qk_n); };
-  auto load_va = [&](int tv, int buf) { VTile::template issue_at<0, VH>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n); };
-  auto load_vb = [&](int tv, int buf) { VTile::template issue_at<VH, VTile::PER>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n); };
+  // With padding, the tiles that reach past the last real row are copied with their row index clamped to it.
+  auto load_k1 = [&](int tk, int buf) {
+    if (TAIL && (tk + 1) * BN > p.n_keys)
+      KTile::issue_clamped(gk1 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF, wave, lane, k_off, qk_n, p.n_keys - 1 - tk * BN);
+    else
+      KTile::issue_at(gk1 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF, wave, lane, k_off, qk_n);
+  };
+  auto load_k2 = [&](int tk, int buf) {
+    if (TAIL && (tk + 1) * BN > p.n_keys)
+      KTile::issue_clamped(gk2 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF + C::K_TILE, wave, lane, k_off, qk_n, p.n_keys - 1 - tk * BN);
+    else
+      KTile::issue_at(gk2 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF + C::K_TILE, wave, lane, k_off, qk_n);
+  };
+  auto load_va = [&](int tv, int buf) {
+    if (TAIL && (tv + 1) * BN > p.n_keys)
+      VTile::template issue_clamped<0, VH>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n, p.n_keys - 1 - tv * BN);
+    else
+      VTile::template issue_at<0, VH>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n);
+  };
+  auto load_vb = [&](int tv, int buf) {
+    if (TAIL && (tv + 1) * BN > p.n_keys)
+      VTile::template issue_clamped<VH, VTile::PER>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n, p.n_keys - 1 - tv * BN);
+    else
+      VTile::template issue_at<VH, VTile::PER>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n);
+  };
 
   // Per-lane LDS byte addresses, computed once.  The XOR swizzle makes the address of a fragment a
   // different function of the lane for every 16-byte chunk column, so there is one register per chunk
@@ -319,7 +348,7 @@ void fwd_kernel(FwdParams p) {
             // registers r, r+1 hold the keys key, key+1 (key even) of this lane's query
             const unsigned query = (unsigned)(qrow0 + 32 * qs);
             const unsigned key = (unsigned)(t * BN + kt * 32 + 8 * (r / 4) + 4 * g + (r % 4));
-            const unsigned word = dropout_word(p.drop, 2u * bh + st, (unsigned)p.N / 2, query >> 1, key >> 1);
+            const unsigned word = dropout_word(dkey, (unsigned)p.N / 2, query >> 1, key >> 1);
             w2 &= (dropout_keep(word, query, key, p.drop.threshold) ? 0x0000ffffu : 0u) |
                   (dropout_keep(word, query, key + 1, p.drop.threshold) ? 0xffff0000u : 0u);
           }
@@ -393,14 +422,16 @@ void fwd_kernel(FwdParams p) {
       }
     (void)qs;
   };
-  auto store_rows = [&](half_t* gbase /* first of this wave's 32 rows */, size_t row_stride) {
+  // `rows`: how many of the wave's 32 rows exist in the destination (32 unless the sequence is padded and
+  // the destination is the caller's tensor, which has no rows past the real length)
+  auto store_rows = [&](half_t* gbase /* first of this wave's 32 rows */, size_t row_stride, int rows) {
     constexpr int LPR = DV / 8;            // lanes per row
     constexpr int RPI = 64 / LPR;          // rows per instruction
 #pragma unroll
     for (int k = 0; k < 32 / RPI; ++k) {
       const int row = k * RPI + lane / LPR, ch = lane % LPR;
       const u32x4 v = *reinterpret_cast<const u32x4*>(stg_own + row * SROW + 8 * ch);
-      *reinterpret_cast<u32x4*>(gbase + (size_t)row * row_stride + 8 * ch) = v;
+      if (!TAIL || row < rows) *reinterpret_cast<u32x4*>(gbase + (size_t)row * row_stride + 8 * ch) = v;
     }
   };
 
@@ -416,7 +447,7 @@ void fwd_kernel(FwdParams p) {
   if (st == 1) stage_rows(0, o[0], inv);
   __syncthreads();
   if (st == 1) {
-    if (p.u2) store_rows(p.u2 + wave_row0 * DV, DV);
+    if (p.u2) store_rows(p.u2 + wave_row0 * DV, DV, 32);
   } else {
     const float lam = da_abi::lambda_of_unit(p, bh);
     const half_t* stg_u2 = smem + (size_t)(wave + NW / 2) * 32 * SROW;
@@ -442,7 +473,8 @@ void fwd_kernel(FwdParams p) {
     }
     stage_rows(0, o[0], scale);
     __builtin_amdgcn_wave_barrier();   // the rows are read back by other lanes of this wave only
-    store_rows(p.y + da_abi::unit_base(p, p.sy, bh) + (size_t)(qt * BM + qw * 32) * (size_t)p.sy.n, (size_t)p.sy.n);
+    store_rows(p.y + da_abi::unit_base(p, p.sy, bh) + (size_t)(qt * BM + qw * 32) * (size_t)p.sy.n, (size_t)p.sy.n,
+               p.n_keys - (qt * BM + qw * 32));
   }
 }
 

@@ -21,9 +21,10 @@ struct FwdParamsT {
   float sm_scale, lambda_init;
   int rms_norm;
   int causal;                   // query i sees keys 0..i only
-  int n_keys;                   // keys n_keys..N-1 are padding and are ignored (N when there is none)
+  int n_keys;                   // rows n_keys..N-1 are padding: ignored as keys, never read from q1..v, never written to y (N when there is none)
   int H;                        // heads per batch entry: unit bh belongs to head bh % H
   int lambda_stride;            // 0: lambda_scale[0] for every head; 1: lambda_scale[head]
+  int lambda_fp32;              // lambda_scale points to fp32 values instead of the tensors' 16-bit type
   Strides sqk, sv, sy;          // layouts of q1,q2,k1,k2 / v / y; u2 and the row statistics are dense
   DropoutCfg drop;               // threshold 0: no dropout
 };
@@ -46,19 +47,23 @@ struct BwdParamsT {
   float sm_scale, lambda_init;
   int rms_norm;
   int causal;
-  int n_keys;                   // keys n_keys..N-1 are padding (N when there is none)
+  int n_keys;                   // rows n_keys..N-1 are padding: ignored as keys, never read from q1..v, y, dy, never written to the gradients
   unsigned stages;              // bit 0 row preprocess, 1 d(lambda) reduce, 2 dK/dV, 3 dQ
   int dlam_fold;                // set by the launcher: extra workgroups at the end of a dK/dV or dQ grid that do the d(lambda) reduce
   int H;                        // heads per batch entry: unit bh belongs to head bh % H
   int lambda_stride;            // 0: one lambda; 1: one per head
-  Strides sqk, sv, sy, sdy;     // layouts of q1,q2,k1,k2 / v / y / dy; everything else is dense
+  int lambda_fp32;              // lambda_scale and dlambda are fp32 instead of the tensors' 16-bit type
+  Strides sqk, sv, sy, sdy;     // layouts of q1,q2,k1,k2 / v / y / dy
+  Strides sdqk, sdv;            // layouts of dq1,dq2,dk1,dk2 / dv; the workspace, u2 and the row statistics are dense [BH,N,.]
   DropoutCfg drop;               // threshold 0: no dropout
 };
 
 // lambda of the (batch, head) unit bh
 template <class P>
 __device__ __forceinline__ float lambda_of_unit(const P& p, int bh) {
-  return (float)p.lambda_scale[(bh % p.H) * p.lambda_stride];
+  const int idx = (bh % p.H) * p.lambda_stride;
+  if (p.lambda_fp32) return reinterpret_cast<const float*>(p.lambda_scale)[idx];
+  return (float)p.lambda_scale[idx];
 }
 
 // offset in elements of the first row of the (batch, head) unit bh

@@ -18,6 +18,8 @@ _FLAG_RMS_NORM = 1      # DIFFATTN_RMS_NORM
 _FLAG_CAUSAL = 2        # DIFFATTN_CAUSAL
 _FLAG_BF16 = 4          # DIFFATTN_BF16
 _FLAG_LAMBDA_PER_HEAD = 8   # DIFFATTN_LAMBDA_PER_HEAD
+_FLAG_LAMBDA_FP32 = 16      # DIFFATTN_LAMBDA_FP32
+_FLAG_UNPADDED = 32         # DIFFATTN_UNPADDED
 _DTYPES = (torch.float16, torch.bfloat16)
 
 
@@ -51,11 +53,6 @@ def _check_inputs(Q1, Q2, K1, K2, V):
     return B, H, N, D
 
 
-def _pad_rows(t, n_pad):
-    """[B,H,N,C] -> dense [B,H,n_pad,C] with zero rows appended."""
-    return torch.nn.functional.pad(t, (0, 0, 0, n_pad - t.size(2)))
-
-
 def _strides_ok(t):
     """Whether the kernels can read t in place: contiguous rows, every other stride a non-negative
     multiple of 8 elements (16-byte aligned rows), base pointer 16-byte aligned."""
@@ -74,18 +71,28 @@ def _is_dense(t):
     return t.stride() == (H * N * C, N * C, C, 1)
 
 
+def _grad_like(t):
+    """An uninitialised gradient buffer in t's memory layout when t is a permuted dense buffer (autograd then
+    takes it as it is instead of copying it into the leaf's layout), else dense."""
+    return torch.empty_like(t)
+
+
 def _current_stream(dev):
     """Raw handle of torch's current stream on dev (no Stream object is built)."""
     return torch._C._cuda_getCurrentRawStream(dev.index if dev.index is not None else torch._C._cuda_getDevice())
 
 
 def _lambda_tensor(lambda_scale, device, dtype=torch.float16, num_heads=1):
-    """The kernels read lambda from device memory (src/kernel.py:138), in the dtype of the tensors.  A
-    python number is wrapped (a superset of the reference, whose float default cannot reach its kernel).
-    A tensor holds one value, like the reference's, or one per head (`num_heads` values, more than one)."""
+    """The kernels read lambda from device memory (src/kernel.py:138).  A python number is wrapped, in the
+    dtype of the tensors (a superset of the reference, whose float default cannot reach its kernel).
+    A tensor holds one value, like the reference's, or one per head (`num_heads` values, more than one);
+    an fp32 tensor is read as fp32 and gets an fp32 gradient, anything else goes through the tensors' dtype
+    like the reference's `dtype=V.dtype` (src/kernel.py:573)."""
     if torch.is_tensor(lambda_scale):
         if lambda_scale.numel() not in (1, num_heads):
             raise ValueError("lambda_scale must have exactly one element, or one per head (%d)" % num_heads)
+        if lambda_scale.dtype == torch.float32:
+            dtype = torch.float32
         return lambda_scale.detach().to(device=device, dtype=dtype).reshape(-1).contiguous()
     return torch.tensor([float(lambda_scale)], dtype=dtype, device=device)
 
@@ -107,24 +114,24 @@ class _diff_attention(torch.autograd.Function):
         dropout = _native.Dropout(dropout_p, int(dropout_seed) & 0xFFFFFFFFFFFFFFFF) if dropout_p > 0 else None
         lib = _native.lib()
         dev = Q1.device
-        # The kernels work on multiples of 128 rows (like the reference's, src/kernel.py:527).  Other
-        # lengths are padded with zero rows here; forward and backward ignore the padding keys, and a
-        # padded query row has a zero upstream gradient, so it adds nothing to dK and dV.
+        # The kernels work on blocks of 128 rows (like the reference's, src/kernel.py:527).  For other lengths
+        # they run on the next multiple of 128, redirect reads past the last real row to that row and ignore
+        # the padding keys: no tensor is padded or copied here; only what the library keeps for itself (u2,
+        # the row statistics, the backward's workspace) is sized for the padded length.
         n_pad = -(-N // _SEQ_MULTIPLE) * _SEQ_MULTIPLE
-        if n_pad != N:
-            q1, q2, k1, k2, v = (_pad_rows(t, n_pad) for t in (Q1, Q2, K1, K2, V))
-        else:
-            # Tensors are read through their strides (the reference passes Q1's and V's to its kernel,
-            # src/kernel.py:487-494): a [B,N,H,d] projection output viewed as [B,H,N,d] is not copied.
-            # The four q/k tensors share one set of strides, as in the reference.
-            q1, q2, k1, k2, v = (_in_place(t) for t in (Q1, Q2, K1, K2, V))
-            if not (q1.stride() == q2.stride() == k1.stride() == k2.stride()):
-                q1, q2, k1, k2 = (t.contiguous() for t in (q1, q2, k1, k2))
+        # Tensors are read through their strides (the reference passes Q1's and V's to its kernel,
+        # src/kernel.py:487-494): a [B,N,H,d] projection output viewed as [B,H,N,d] is not copied.
+        # The four q/k tensors share one set of strides, as in the reference.
+        q1, q2, k1, k2, v = (_in_place(t) for t in (Q1, Q2, K1, K2, V))
+        if not (q1.stride() == q2.stride() == k1.stride() == k2.stride()):
+            q1, q2, k1, k2 = (t.contiguous() for t in (q1, q2, k1, k2))
         lam = _lambda_tensor(LAMBDA_SCALE, dev, Q1.dtype, H)
         rms_norm = bool(rms_norm)
         flags = ((_FLAG_RMS_NORM if rms_norm else 0) | (_FLAG_CAUSAL if causal else 0)
                  | (_FLAG_BF16 if Q1.dtype == torch.bfloat16 else 0)
-                 | (_FLAG_LAMBDA_PER_HEAD if lam.numel() > 1 else 0))
+                 | (_FLAG_LAMBDA_PER_HEAD if lam.numel() > 1 else 0)
+                 | (_FLAG_LAMBDA_FP32 if lam.dtype == torch.float32 else 0)
+                 | (_FLAG_UNPADDED if n_pad != N else 0))
 
         y = torch.empty_like(v)         # v's layout when v is a permuted dense buffer, else dense
         layout = None
@@ -159,25 +166,22 @@ class _diff_attention(torch.autograd.Function):
         ctx.SM_SCALE = float(SM_SCALE)
         ctx.LAMBDA_INIT = float(LAMBDA_INIT)
         ctx.FLAGS = flags
-        ctx.N_VALID = N
+        ctx.N_PAD = n_pad
         ctx.DROPOUT = dropout
         ctx.lambda_meta = (LAMBDA_SCALE.dtype, LAMBDA_SCALE.shape) if torch.is_tensor(LAMBDA_SCALE) else None
-        return y if n_pad == N else y[:, :, :N].contiguous()
+        return y
 
     @staticmethod
     @once_differentiable        # the gradients are plain kernel outputs: a second derivative raises
     def backward(ctx, dO):
         q1, q2, k1, k2, v, y, u2, lse1, lse2, rinv, lam = ctx.saved_tensors
-        B, H, N, D = q1.shape           # N is the padded length here
+        B, H, N, D = q1.shape
+        n_pad = ctx.N_PAD
         lib = _native.lib()
         dev = q1.device
-        n_valid = ctx.N_VALID
         if dO.dtype != q1.dtype:
             dO = dO.to(q1.dtype)
-        dO = _pad_rows(dO, N) if n_valid != N else _in_place(dO)
-        layout = None
-        if not (_is_dense(q1) and _is_dense(v) and _is_dense(y) and _is_dense(dO)):
-            layout = _native.Layout(*q1.stride()[:3], *v.stride()[:3], *y.stride()[:3], *dO.stride()[:3])
+        dO = _in_place(dO)
 
         # only the kernels whose outputs some input asked for are launched (stage bits of the C ABI:
         # 1 row preprocess, 2 d(lambda) reduction, 4 dK/dV, 8 dQ)
@@ -185,19 +189,21 @@ class _diff_attention(torch.autograd.Function):
         want_q, want_kv = need[0] or need[1], need[2] or need[3] or need[4]
         want_lam = ctx.lambda_meta is not None and need[6]
         stages = 1 | (2 if want_lam else 0) | (4 if want_kv else 0) | (8 if want_q else 0)
-        # gradients are dense [B,H,N,.] whatever the layout of the inputs; those of equal shape share
-        # one allocation
+        # Gradients are written in the memory layout of the tensors they belong to (autograd would otherwise
+        # copy each one into its leaf's layout).  The four q/k gradients share one set of strides, like q1..k2.
         dq1 = dq2 = dk1 = dk2 = dv = None
-        n_qk = (2 if want_q else 0) + (2 if want_kv else 0)
-        if n_qk:
-            gqk = torch.empty((n_qk, B, H, N, D), device=dev, dtype=q1.dtype)
-            if want_q:
-                dq1, dq2 = gqk[0], gqk[1]
-            if want_kv:
-                dk1, dk2 = gqk[n_qk - 2], gqk[n_qk - 1]
-                dv = torch.empty((B, H, N, 2 * D), device=dev, dtype=q1.dtype)
-        dlam = torch.empty(lam.numel(), device=dev, dtype=q1.dtype) if want_lam else None
-        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, N, D, ctx.FLAGS)
+        if want_q:
+            dq1, dq2 = _grad_like(q1), _grad_like(q1)
+        if want_kv:
+            dk1, dk2, dv = _grad_like(q1), _grad_like(q1), _grad_like(v)
+        gqk = dq1 if want_q else dk1        # (a view that is not a permuted dense buffer gets a dense gradient)
+        layout = None
+        if not (_is_dense(q1) and _is_dense(v) and _is_dense(y) and _is_dense(dO)):
+            layout = _native.Layout(*q1.stride()[:3], *v.stride()[:3], *y.stride()[:3], *dO.stride()[:3],
+                                    *(gqk.stride()[:3] if gqk is not None else (0, 0, 0)),
+                                    *(dv.stride()[:3] if dv is not None else (0, 0, 0)))
+        dlam = torch.empty(lam.numel(), device=dev, dtype=lam.dtype) if want_lam else None
+        ws_bytes = lib.diffattn_backward_workspace_bytes(B, H, n_pad, D, ctx.FLAGS)
         ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
 
         def launch():
@@ -205,7 +211,7 @@ class _diff_attention(torch.autograd.Function):
                 q1.data_ptr(), q2.data_ptr(), k1.data_ptr(), k2.data_ptr(), v.data_ptr(), lam.data_ptr(),
                 y.data_ptr(), u2.data_ptr(), lse1.data_ptr(), lse2.data_ptr(), _ptr(rinv), dO.data_ptr(),
                 _ptr(dq1), _ptr(dq2), _ptr(dk1), _ptr(dk2), _ptr(dv), _ptr(dlam),
-                ws.data_ptr(), ws_bytes, B, H, N, n_valid, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stages,
+                ws.data_ptr(), ws_bytes, B, H, n_pad, N, D, ctx.SM_SCALE, ctx.LAMBDA_INIT, ctx.FLAGS, stages,
                 layout, ctx.DROPOUT, _current_stream(dev))
 
         if dev.index is not None and dev.index != torch._C._cuda_getDevice():
@@ -219,8 +225,5 @@ class _diff_attention(torch.autograd.Function):
         if want_lam:
             dtype, shape = ctx.lambda_meta
             dlambda = dlam.to(dtype).reshape(shape)
-        if n_valid != N:
-            dq1, dq2, dk1, dk2, dv = (None if t is None else t[:, :, :n_valid].contiguous()
-                                      for t in (dq1, dq2, dk1, dk2, dv))
         # one slot per forward argument: nine, or more when causal / dropout arguments were passed
         return (dq1, dq2, dk1, dk2, dv, None, dlambda) + (None,) * (len(ctx.needs_input_grad) - 7)

@@ -32,12 +32,19 @@ def MultiheadDiffAttnKernel(
     src/kernel.py:4) lets query i attend to keys 0..i only.  `dropout_p` (likewise missing in the
     reference) drops every entry of each of the two softmax maps independently with that
     probability, in steps of 1/256, and scales the kept ones by 1/(1-p); the masks are a function of
-    `dropout_seed` (drawn from torch's default generator when None) and the position.
+    `dropout_seed` (drawn from torch's default CPU generator when None) and the position.  The seed
+    travels as a launch argument: a HIP graph captured around the call replays the same masks, so a call
+    under capture has to name its seed.
     """
     head_dim = q1.size(-1)
     sm_scale = 1 / math.sqrt(head_dim)
     if dropout_p:
         if dropout_seed is None:
+            # The seed is a host value handed to the kernels with the launch: under stream capture it would be
+            # frozen into the graph and every replay would drop the same entries.
+            if q1.is_cuda and torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("dropout under stream capture needs an explicit dropout_seed (the same masks are "
+                                   "then applied on every replay of the graph)")
             dropout_seed = int(torch.randint(0, 2 ** 62, (1,)).item())
         return _diff_attention.apply(q1, q2, k1, k2, v, sm_scale, lambda_scale, lambda_init, rms_norm, bool(causal),
                                      float(dropout_p), int(dropout_seed))

@@ -66,7 +66,9 @@ class DiffAttn(nn.Module):
         q = self.q_proj(x).view(B, N, H, 2, d).permute(3, 0, 2, 1, 4)
         k = self.k_proj(x).view(B, N, H, 2, d).permute(3, 0, 2, 1, 4)
         v = self.v_proj(x).view(B, N, H, 2 * d).transpose(1, 2)
-        lam = self.lambda_scale().to(x.dtype)
+        # lambda stays in fp32: the operator then reads it unrounded and returns its gradient in fp32, which a
+        # gradient scaler's loss scale cannot push out of range
+        lam = self.lambda_scale()
         # views of the projection outputs: the operator reads them through their strides and returns the
         # heads in v's [B,N,H,2d] memory layout, so neither side of it copies
         heads = self.attention(q[0], q[1], k[0], k[1], v, lambda_scale=lam, lambda_init=self.lambda_init, rms_norm=True,
