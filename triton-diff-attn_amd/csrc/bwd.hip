@@ -350,7 +350,9 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   struct Scores { f16v s1, s2, dp; };
   struct Packed { h8 pc[2], d1[2], d2[2]; };   // A operands of the dV / dK1 / dK2 products
   constexpr int NPROD = 2 * NKS + (DO_K ? NKV : 0);   // score products per sub-tile (dP is needed for dK only)
-  constexpr int DEPTH = DROP ? 1 : 3;          // A fragments requested ahead of their product (dropout: registers are short)
+  // the D = 128 instantiations with dropout are short of registers: they request one fragment ahead
+  constexpr bool kShort = DROP && D == 128;
+  constexpr int DEPTH = kShort ? 1 : 3;        // A fragments requested ahead of their product
 
   // Product k of a sub-tile: even k is k-step k/2 of dP, odd k alternates k-steps of S1 and S2, so
   // the three accumulation chains advance together; without dP (MODE 1) S1 and S2 alternate.
@@ -362,16 +364,17 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     }
     return lds_h8(xb[k >> 1], buf * C::XBUF + qs * 32 * DV * 2);
   };
-  // The dropout instantiations spill a few registers; there the products are issued as ordinary
-  // (compiler-visible) matrix instructions, so that the compiler places every wait state itself:
-  // with reloads of spilled fragments in front of them the opaque assembly form read stale operands.
+  // The products read their resident operand from AGPRs through the inline-assembly form.  That form is
+  // safe only while nothing is spilled (a reloaded operand directly in front of it would be read too early);
+  // the build checks that no backward kernel uses scratch memory.  The register-short instantiations issue
+  // ordinary (compiler-visible) matrix instructions, for which the compiler places every wait state itself.
   auto prod_mfma = [&](int k, h8 a, Scores& out) {
     if (!DO_K || (k & 1)) {
       const int t = DO_K ? (k >> 1) : k, ks = t >> 1;
-      if (t & 1) out.s2 = DROP ? mfma32(a, kf2[ks], out.s2) : mfma32_bagpr(a, kf2[ks], out.s2);
-      else       out.s1 = DROP ? mfma32(a, kf1[ks], out.s1) : mfma32_bagpr(a, kf1[ks], out.s1);
+      if (t & 1) out.s2 = kShort ? mfma32(a, kf2[ks], out.s2) : mfma32_bagpr(a, kf2[ks], out.s2);
+      else       out.s1 = kShort ? mfma32(a, kf1[ks], out.s1) : mfma32_bagpr(a, kf1[ks], out.s1);
     } else {
-      out.dp = DROP ? mfma32(a, vf[k >> 1], out.dp) : mfma32_bagpr(a, vf[k >> 1], out.dp);
+      out.dp = kShort ? mfma32(a, vf[k >> 1], out.dp) : mfma32_bagpr(a, vf[k >> 1], out.dp);
     }
   };
   // Row statistics written by the preprocess kernel: 0: -lse1*log2e, 1: -lse2*log2e, 2: -delta1,
@@ -512,7 +515,7 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
   // of the step and read during the second, its upper half is written during the second half and
   // read during the first half of the next step.
   static_assert(NPROD % 16 == 0 || 16 % NPROD == 0, "rows are spread evenly over the products");
-  constexpr int AHEAD = DROP ? 1 : 3;          // B fragments requested ahead of their product
+  constexpr int AHEAD = kShort ? 1 : 3;        // B fragments requested ahead of their product
   auto fused = [&](int bufn, int qsn, Scores& s_nxt, int bufc, int qsc, const Scores& s_cur, Packed& pk,
                    int bufp, int qsp, int tile_next, auto buf_next_tag, auto fetch_tag, auto masked_tag, int rel, int qbase) {
     constexpr int buf_next = decltype(buf_next_tag)::value;
