@@ -127,16 +127,17 @@ def test_host_validation_errors():
     assert _lambda_tensor(torch.tensor([[0.1], [0.2], [0.3]]), torch.device("cpu"), num_heads=3).dtype == torch.float32
     assert _lambda_tensor(torch.tensor([0.5], dtype=torch.float64), torch.device("cpu"), torch.bfloat16).dtype == torch.bfloat16
     assert _lambda_tensor(0.5, torch.device("cpu"), torch.bfloat16).dtype == torch.bfloat16
-    from kernel import _pad_rows
+    from kernel import _grad_like, _in_place, _is_dense, _strides_ok
     x = torch.arange(2 * 3 * 5 * 4, dtype=torch.float16).reshape(2, 3, 5, 4)
-    padded = _pad_rows(x, 8)
-    assert padded.shape == (2, 3, 8, 4) and padded.is_contiguous()
-    assert torch.equal(padded[:, :, :5], x) and padded[:, :, 5:].abs().sum() == 0
-    from kernel import _in_place, _is_dense, _strides_ok
     wide = torch.zeros(2, 16, 3, 64, dtype=torch.float16)              # a [B,N,H,C] buffer seen as [B,H,N,C]
     view = wide.transpose(1, 2)
     assert _strides_ok(view) and _in_place(view) is view and not _is_dense(view) and _is_dense(wide)
     assert not _strides_ok(x.transpose(2, 3)) and _in_place(x.transpose(2, 3)).is_contiguous()    # last dim strided
+    # a gradient buffer takes the layout of a permuted dense tensor; for a slice of a longer tensor it is a
+    # compact buffer in the same dimension order: either way its own strides go to the kernels
+    assert _grad_like(view).stride() == view.stride()
+    sliced = _grad_like(wide[:, :8].transpose(1, 2)[:, :, :, :32])
+    assert _strides_ok(sliced) and sliced.stride() == (8 * 3 * 32, 32, 3 * 32, 1)
     assert not _strides_ok(torch.zeros(2, 3, 5, 36, dtype=torch.float16)[..., :32])               # rows not 16-byte aligned
     lam = _lambda_tensor(0.25, torch.device("cpu"))
     assert lam.dtype == torch.float16 and lam.shape == (1,) and lam.item() == 0.25

@@ -28,18 +28,39 @@ def test_scanner_flags_a_write_right_before_an_asm_mfma():
     assert isa_scan.registers("v[2:4], a7, s[0:1], v10") == {"v2", "v3", "v4", "a7", "v10"}
 
 
-@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
-@pytest.mark.parametrize("variant", [[], ["-DDA_BF16"]], ids=["fp16", "bf16"])
-def test_backward_kernels_have_no_unprotected_asm_mfma(tmp_path, variant):
+def _load_build():
     import importlib.util
     spec = importlib.util.spec_from_file_location("da_build", os.path.join(ROOT, "triton-diff-attn_amd", "build.py"))
     build = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(build)
-    out = tmp_path / "bwd.s"
-    cmd = [build.HIPCC] + [f for f in build.FLAGS if f != "-fPIC"] + variant + ["--cuda-device-only", "-S", "-o", str(out),
-                                                                          os.path.join(CSRC, "bwd.hip")]
-    subprocess.run(cmd, check=True, capture_output=True)
-    text = out.read_text()
+    return build
+
+
+@pytest.fixture(scope="module")
+def assembly(tmp_path_factory):
+    """Assembly text of the three compilations the tests below read (backward fp16 and bf16, forward fp16),
+    compiled side by side."""
+    build = _load_build()
+    tmp = tmp_path_factory.mktemp("isa")
+    jobs = {}
+    for key, src, variant in (("bwd_fp16", "bwd.hip", []), ("bwd_bf16", "bwd.hip", ["-DDA_BF16"]), ("fwd_fp16", "fwd.hip", [])):
+        out = tmp / (key + ".s")
+        cmd = [build.HIPCC] + [f for f in build.FLAGS if f != "-fPIC"] + variant + ["--cuda-device-only", "-S", "-o", str(out),
+                                                                              os.path.join(CSRC, src)]
+        jobs[key] = (out, subprocess.Popen(cmd, stdout=subprocess.DEVNULL, stderr=subprocess.PIPE))
+    texts = {}
+    for key, (out, proc) in jobs.items():
+        _, err = proc.communicate()
+        assert proc.returncode == 0, err.decode()[-2000:]
+        texts[key] = out.read_text()
+    return texts
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+@pytest.mark.parametrize("variant", ["fp16", "bf16"])
+def test_backward_kernels_have_no_unprotected_asm_mfma(assembly, variant):
+    text = assembly["bwd_" + variant]
+    variant = variant == "bf16"
     assert ("v_mfma_f32_32x32x16_bf16" if variant else "v_mfma_f32_32x32x16_f16") in text and ";;#ASMSTART" in text
     hazards = isa_scan.asm_mfma_hazards(text)
     assert hazards == [], "VALU write right before an inline-asm MFMA: %s" % hazards[:5]
@@ -53,22 +74,14 @@ def test_backward_kernels_have_no_unprotected_asm_mfma(tmp_path, variant):
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
-def test_forward_kernels_do_not_spill_in_their_loops(tmp_path):
+def test_forward_kernels_do_not_spill_in_their_loops(assembly):
     """The forward instantiations without dropout use no scratch memory at all; those with dropout may
     park a value across the main loop, but never inside it."""
-    import importlib.util
     import re
-    spec = importlib.util.spec_from_file_location("da_build", os.path.join(ROOT, "triton-diff-attn_amd", "build.py"))
-    build = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(build)
-    out = tmp_path / "fwd.s"
-    cmd = [build.HIPCC] + [f for f in build.FLAGS if f != "-fPIC"] + ["--cuda-device-only", "-S", "-o", str(out),
-                                                                      os.path.join(CSRC, "fwd.hip")]
-    subprocess.run(cmd, check=True, capture_output=True)
-    kernels = re.findall(r"^(_Z\w*fwd_kernel\w*):[^\n]*\n(.*?)s_endpgm", out.read_text(), re.S | re.M)
-    assert len(kernels) == 36
+    kernels = re.findall(r"^(_Z\w*fwd_kernel\w*):[^\n]*\n(.*?)s_endpgm", assembly["fwd_fp16"], re.S | re.M)
+    assert len(kernels) == 40          # D x rms_norm x mask x dropout, plus the 64-row variants of the plain ones at D <= 64
     for name, body in kernels:
-        dropout = name.split("EEEv")[0].endswith("Lb1")
+        dropout = re.search(r"fwd_kernelILi\d+ELb\dELi\dELb(\d)", name).group(1) == "1"
         if not dropout:
             assert "scratch_" not in body, name
             continue
@@ -83,16 +96,13 @@ def test_forward_kernels_do_not_spill_in_their_loops(tmp_path):
 
 def test_build_rejects_a_spilling_kernel():
     """build.py reads the compiler's per-kernel resource remarks and refuses kernels that must not spill."""
-    import importlib.util
-    spec = importlib.util.spec_from_file_location("da_build", os.path.join(ROOT, "triton-diff-attn_amd", "build.py"))
-    build = importlib.util.module_from_spec(spec)
-    spec.loader.exec_module(build)
+    build = _load_build()
     remark = ("x.hip:1:1: remark: Function Name: %s [-Rpass-analysis=kernel-resource-usage]\n"
               "x.hip:1:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]\n"
               "x.hip:1:1: remark:     ScratchSize [bytes/lane]: %d [-Rpass-analysis=kernel-resource-usage]\n")
     dkdv = "_ZN2da15bwd_dkdv_kernelILi64ELi0ELb0ELb0EEEvN6da_abi10BwdParamsTIDF16_EE"
-    fwd_plain = "_ZN2da10fwd_kernelILi64ELb1ELi0ELb0EEEvN6da_abi10FwdParamsTIDF16_EE"
-    fwd_drop = "_ZN2da10fwd_kernelILi64ELb1ELi1ELb1EEEvN6da_abi10FwdParamsTIDF16_EE"
+    fwd_plain = "_ZN2da10fwd_kernelILi64ELb1ELi0ELb0ELb1EEEvN6da_abi10FwdParamsTIDF16_EE"
+    fwd_drop = "_ZN2da10fwd_kernelILi64ELb1ELi1ELb1ELb0EEEvN6da_abi10FwdParamsTIDF16_EE"
     build.check_resources("x.hip", remark % (dkdv, 0) + remark % (fwd_plain, 0) + remark % (fwd_drop, 24))
     for name in (dkdv, fwd_plain):
         with pytest.raises(RuntimeError, match="must not spill"):

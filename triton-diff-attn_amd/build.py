@@ -38,7 +38,8 @@ def check_resources(src, remarks):
     for name, scratch in re.findall(r"Function Name: (\S+).*?ScratchSize \[bytes/lane\]: (\d+)", remarks, re.S):
         if int(scratch) == 0:
             continue
-        dropout = name.split("EEEv")[0].endswith("Lb1")
+        m = re.search(r"fwd_kernelILi\d+ELb\dELi\dELb(\d)", name)       # <D, RMS, MASK, DROP, ...>
+        dropout = bool(m) and m.group(1) == "1"
         if "bwd_" in name or ("fwd_kernel" in name and not dropout):
             bad.append("%s: %s bytes of scratch per lane" % (name, scratch))
     if bad:

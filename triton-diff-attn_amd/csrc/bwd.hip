@@ -115,25 +115,26 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
 
 // Output o of n_out is the sum of the partials of the units o, o + n_out, o + 2 n_out, ...: with n_out = 1
 // every unit (one lambda), with n_out = H the units of head o (one lambda per head).  `per_unit`
-// consecutive partials belong to a unit.  One workgroup per output; its first 256 threads add in a fixed
-// order whatever the size of the workgroup, so the result does not depend on the kernel that hosts it.
+// consecutive partials belong to a unit.  One workgroup per output.  The sum is formed over 256 slots and a
+// binary tree in a fixed order; a workgroup of fewer threads lets each thread play several slots, so the
+// result does not depend on the kernel that hosts the reduction.
 __device__ __forceinline__ void dlambda_reduce(const float* __restrict__ part, int per_unit, int n_units, half_t* out,
                                                int o, int n_out, float* red, int out_fp32) {
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, nt = blockDim.x;
   const int n = (n_units / n_out) * per_unit;        // partials this workgroup sums
-  float acc = 0.f;
-  if (tid < 256) {
+  for (int slot = tid; slot < 256; slot += nt) {
+    float acc = 0.f;
     if (n_out == 1) {
-      for (int i = tid; i < n; i += 256) acc += part[i];
+      for (int i = slot; i < n; i += 256) acc += part[i];
     } else {
-      for (int i = tid; i < n; i += 256) acc += part[(size_t)(o + (i / per_unit) * n_out) * per_unit + i % per_unit];
+      for (int i = slot; i < n; i += 256) acc += part[(size_t)(o + (i / per_unit) * n_out) * per_unit + i % per_unit];
     }
-    red[tid] = acc;
+    red[slot] = acc;
   }
   __syncthreads();
 #pragma unroll
   for (int s = 128; s >= 1; s >>= 1) {
-    if (tid < s) red[tid] += red[tid + s];
+    for (int slot = tid; slot < s; slot += nt) red[slot] += red[slot + s];
     __syncthreads();
   }
   if (tid == 0) {
@@ -160,10 +161,10 @@ __global__ __launch_bounds__(256) void bwd_dlambda_kernel(const float* __restric
   }
 
 // ------------------------------------------------------------------------------------------------
-template <int D>
+template <int D, int NWAVES = 4>
 struct DkvCfg {
   static constexpr int DV = 2 * D;
-  static constexpr int NW = 4;                 // waves per workgroup, 32 keys each
+  static constexpr int NW = NWAVES;            // waves per workgroup, 32 keys each (2: half-size key blocks for small grids)
   static constexpr int NT = NW * 64;
   static constexpr int BK = NW * 32;           // keys per workgroup
   static constexpr int BQ = (D <= 64) ? 64 : 32;  // query rows per staged tile
@@ -197,9 +198,9 @@ struct DkvCfg {
 // PADDED: rows n_keys..N-1 are padding.  As queries they read the last real row of Q1 and Q2 (the row the
 // forward used for their logsumexp) and carry dX = 0; as keys they read the last real row of K1, K2, V and
 // their results are not stored.
-template <int D, int MODE, bool CAUSAL, bool DROP, bool PADDED>
-__global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_kernel(BwdParams p) {
-  using C = DkvCfg<D>;
+template <int D, int MODE, bool CAUSAL, bool DROP, bool PADDED, int NWAVES = 4>
+__global__ __launch_bounds__((DkvCfg<D, NWAVES>::NT)) __attribute__((amdgpu_waves_per_eu(1, 1))) void bwd_dkdv_kernel(BwdParams p) {
+  using C = DkvCfg<D, NWAVES>;
   constexpr int DV = C::DV, NW = C::NW, BK = C::BK, BQ = C::BQ;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32, NVT = DV / 32;
   constexpr bool DO_V = (MODE != 2), DO_K = (MODE != 1);
@@ -364,17 +365,19 @@ __global__ __launch_bounds__(DkvCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(1
     }
     return lds_h8(xb[k >> 1], buf * C::XBUF + qs * 32 * DV * 2);
   };
-  // The products read their resident operand from AGPRs through the inline-assembly form.  That form is
-  // safe only while nothing is spilled (a reloaded operand directly in front of it would be read too early);
-  // the build checks that no backward kernel uses scratch memory.  The register-short instantiations issue
-  // ordinary (compiler-visible) matrix instructions, for which the compiler places every wait state itself.
+  // The products read their resident operand from AGPRs through the inline-assembly form, for which the
+  // compiler places no wait states: nothing may be spilled (a reloaded operand directly in front of such a
+  // product would be read too early; the build checks that no backward kernel uses scratch memory) and no
+  // VALU instruction may write an operand right in front of one (an assembly scan in the tests checks that).
+  // The dropout instantiations, whose mask arithmetic makes the compiler shuffle operands, issue ordinary
+  // (compiler-visible) matrix instructions instead: the compiler then places every wait state itself.
   auto prod_mfma = [&](int k, h8 a, Scores& out) {
     if (!DO_K || (k & 1)) {
       const int t = DO_K ? (k >> 1) : k, ks = t >> 1;
-      if (t & 1) out.s2 = kShort ? mfma32(a, kf2[ks], out.s2) : mfma32_bagpr(a, kf2[ks], out.s2);
-      else       out.s1 = kShort ? mfma32(a, kf1[ks], out.s1) : mfma32_bagpr(a, kf1[ks], out.s1);
+      if (t & 1) out.s2 = DROP ? mfma32(a, kf2[ks], out.s2) : mfma32_bagpr(a, kf2[ks], out.s2);
+      else       out.s1 = DROP ? mfma32(a, kf1[ks], out.s1) : mfma32_bagpr(a, kf1[ks], out.s1);
     } else {
-      out.dp = kShort ? mfma32(a, vf[k >> 1], out.dp) : mfma32_bagpr(a, vf[k >> 1], out.dp);
+      out.dp = DROP ? mfma32(a, vf[k >> 1], out.dp) : mfma32_bagpr(a, vf[k >> 1], out.dp);
     }
   };
   // Row statistics written by the preprocess kernel: 0: -lse1*log2e, 1: -lse2*log2e, 2: -delta1,
@@ -996,6 +999,13 @@ static hipError_t launch_bwd_t(const BwdParams& p_in, hipStream_t stream) {
   BwdParams p = p_in;
   const int n_prep = bwd_num_partials(p.BH, p.N, D);
   hipError_t e = hipSuccess;
+  // Shape-aware launch geometry (the reference autotunes its tiles per (N, D, Dv), src/kernel.py:12-19): a problem
+  // whose 128-row blocks do not fill the chip once runs in twice as many 64-row workgroups.  A pure function of
+  // (B*H, N, D) and the options: no tuning state.  Only the plain dK/dV instantiation has the small variant
+  // (the dQ kernel was measured with 64-row workgroups too: 15-20 % slower on such grids, so it keeps 128).
+  constexpr int kNumCU = 256;
+  const bool small_grid = D != 128 && !p.causal && !p.drop.threshold && p.n_keys == p.N &&
+                          (long long)p.BH * (p.N / 128) < kNumCU;
   // the d(lambda) reduce rides in the first dK/dV or dQ launch when there is one, else it is a launch of its own
   const int n_lambda = p.lambda_stride ? p.H : 1;
   bool fold = (p.stages & 2u) && (p.stages & 12u);
@@ -1012,7 +1022,15 @@ static hipError_t launch_bwd_t(const BwdParams& p_in, hipStream_t stream) {
                        p.dlam_part, n_prep / p.BH, p.BH, p.dlambda, p.lambda_fp32);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
-  if (p.stages & 4u) {
+  if ((p.stages & 4u) && small_grid) {
+    if constexpr (D != 128) {
+      p.dlam_fold = fold ? n_lambda : 0;
+      fold = false;
+      const dim3 grid(p.BH * (p.N / DkvCfg<D, 2>::BK) + p.dlam_fold), block(DkvCfg<D, 2>::NT);
+      hipLaunchKernelGGL((bwd_dkdv_kernel<D, 0, false, false, false, 2>), grid, block, 0, stream, p);
+      if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
+  } else if (p.stages & 4u) {
     const dim3 block(DkvCfg<D>::NT);
     auto launch_mode = [&](auto mode_tag) {
       constexpr int M = decltype(mode_tag)::value;
@@ -1046,7 +1064,6 @@ static hipError_t launch_bwd_t(const BwdParams& p_in, hipStream_t stream) {
     // runs one wave per SIMD and therefore always has four waves).  A grid so small that even its
     // 128-row workgroups all fit on the chip at once is launched that way too: it finishes sooner
     // in twice as many, half as long workgroups.
-    constexpr int kNumCU = 256;
     bool wide = false;
     auto launch_dq = [&](auto nw_tag, dim3 grid, dim3 block) {
       constexpr int NWV = decltype(nw_tag)::value;

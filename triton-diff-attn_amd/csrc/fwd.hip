@@ -18,14 +18,15 @@
 
 namespace DA_NS {
 
-template <int D>
+// SMALL: 64 query rows per workgroup at D <= 64 as well, for problems whose 128-row blocks do not fill the chip.
+template <int D, bool SMALL = false>
 struct FwdCfg {
   static constexpr int DV = 2 * D;
   static constexpr int BN = (D <= 64) ? 64 : 32;   // keys per tile
   static constexpr int QS = 1;                     // 32-row query blocks per wave
   // query rows per workgroup; the output accumulators of a D = 128 wave need more than 256
   // registers, so those workgroups have four waves at one wave per SIMD
-  static constexpr int BM = (D == 128) ? 64 : 128;
+  static constexpr int BM = (D == 128 || SMALL) ? 64 : 128;
   static constexpr int NW = 2 * BM / (32 * QS);    // waves per workgroup: half of them per softmax stream
   static constexpr int NT = NW * 64;
   static constexpr int OCC = (QS == 2 || D == 128) ? 1 : 2;   // waves per SIMD the register budget is sized for
@@ -50,10 +51,10 @@ constexpr float kRescaleThreshold = 8.0f;   // log2 units: probabilities stay be
 // DROP: dropout on both softmax maps (not in the reference, which lists it as missing,
 // src/kernel.py:4): a dropped probability still counts in its row's sum but not in P*V, and the
 // kept ones are scaled by 1/(1-p) -- in the epilogue, together with 1/l.
-template <int D, bool RMS, int MASK, bool DROP>
-__global__ __launch_bounds__(FwdCfg<D>::NT) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::OCC, FwdCfg<D>::OCC)))
+template <int D, bool RMS, int MASK, bool DROP, bool SMALL = false>
+__global__ __launch_bounds__((FwdCfg<D, SMALL>::NT)) __attribute__((amdgpu_waves_per_eu(FwdCfg<D, SMALL>::OCC, FwdCfg<D, SMALL>::OCC)))
 void fwd_kernel(FwdParams p) {
-  using C = FwdCfg<D>;
+  using C = FwdCfg<D, SMALL>;
   constexpr int DV = C::DV, BN = C::BN, NW = C::NW, BM = C::BM, QS = C::QS;
   constexpr int NKS = D / 16;                // k-steps of the score product
   constexpr int NKT = BN / 32;               // 32-key tiles of S^T
@@ -137,7 +138,7 @@ void fwd_kernel(FwdParams p) {
   // causal: keys beyond the last row of the workgroup are never visited (BM is a multiple of 2*BN,
   // so the tile count stays even)
   const int n_tiles = CAUSAL ? (qt + 1) * (BM / BN) : p.N / BN;
-  static_assert(BM % (2 * BN) == 0, "an even number of key tiles per query block");
+  static_assert(!CAUSAL || BM % (2 * BN) == 0, "an even number of key tiles per query block");
   constexpr int VH = (VTile::PER + 1) / 2;   // V instructions are issued in two groups
   const unsigned k_off = KTile::lane_off(wave, lane, qk_n), v_off = VTile::lane_off(wave, lane, v_n);
   // With padding, the tiles that reach past the last real row are copied with their row index clamped to it.
@@ -492,6 +493,18 @@ template <int D>
 static hipError_t launch_fwd_t(const FwdParams& p, hipStream_t stream) {
   dim3 grid(p.BH * (p.N / FwdCfg<D>::BM)), block(FwdCfg<D>::NT);
   const bool drop = p.drop.threshold != 0;
+  // Shape-aware launch geometry (the reference autotunes its tiles per (N, D, Dv), src/kernel.py:12-19): a problem
+  // whose 128-row blocks do not fill the chip once runs in twice as many 64-row workgroups.  A pure function of
+  // (B*H, N, D) and the options: no tuning state.  Only the plain instantiations have the small variant.
+  constexpr int kNumCU = 256;
+  if constexpr (D != 128) {
+    if (!p.causal && !drop && p.n_keys == p.N && (long long)p.BH * (p.N / 128) < kNumCU) {
+      const dim3 sgrid(p.BH * (p.N / FwdCfg<D, true>::BM)), sblock(FwdCfg<D, true>::NT);
+      if (p.rms_norm) hipLaunchKernelGGL((fwd_kernel<D, true, 0, false, true>), sgrid, sblock, 0, stream, p);
+      else            hipLaunchKernelGGL((fwd_kernel<D, false, 0, false, true>), sgrid, sblock, 0, stream, p);
+      return hipGetLastError();
+    }
+  }
   if (p.rms_norm) {
     if (drop) launch_fwd_c<D, true, true>(p, grid, block, stream);
     else      launch_fwd_c<D, true, false>(p, grid, block, stream);
