@@ -37,6 +37,9 @@ struct FwdCfg {
   // the loop can be unrolled over one turn of the ring with every buffer known at compile time: an LDS
   // address is then a per-lane register plus an immediate offset, with no arithmetic inside the loop.
   static constexpr int NBUF = 4;
+  // A barrier every second tile instead of every tile (the ring allows it): measured in one GPU call,
+  // 3.3 % faster at D = 32, 3 % slower at D = 64 and 5 % slower at D = 128.
+  static constexpr bool PAIR = (D == 32);
   static constexpr int KBUF_BYTES = K_BUF * 2, VBUF_BYTES = V_TILE * 2, VBASE_BYTES = NBUF * KBUF_BYTES;
   static_assert(NBUF * KBUF_BYTES <= 65536 && NBUF * VBUF_BYTES <= 65536, "immediate offsets reach every buffer");
   static constexpr int TILES = NBUF * (K_BUF + V_TILE);
@@ -381,8 +384,14 @@ void fwd_kernel(FwdParams p) {
     }
 
     // the tiles needed next were requested one iteration ago: only this iteration's loads may remain
-    wait_async_tiles_except(loads_per_iter);
-    __syncthreads();
+    if constexpr (C::PAIR) {
+      // the ring of four lets the workgroup meet every second tile only: the copies for the next two tiles
+      // (requested during the last two) have landed for everybody, and the last two buffers may be refilled
+      if constexpr (POS & 1) { wait_async_tiles(); __syncthreads(); }
+    } else {
+      wait_async_tiles_except(loads_per_iter);
+      __syncthreads();
+    }
   };
 
   // the tile count is even (N is a multiple of 128, tiles are at most 64 keys)
