@@ -145,30 +145,33 @@ void fwd_kernel(FwdParams p) {
   constexpr int VH = (VTile::PER + 1) / 2;   // V instructions are issued in two groups
   const unsigned k_off = KTile::lane_off(wave, lane, qk_n), v_off = VTile::lane_off(wave, lane, v_n);
   // With padding, the tiles that reach past the last real row are copied with their row index clamped to it.
-  auto load_k1 = [&](int tk, int buf) {
-    if (TAIL && (tk + 1) * BN > p.n_keys)
+  // `tail` (a compile-time tag) says whether the call site can meet such a tile at all.
+  auto load_k1 = [&](int tk, int buf, auto tail) {
+    if (TAIL && decltype(tail)::value && (tk + 1) * BN > p.n_keys)
       KTile::issue_clamped(gk1 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF, wave, lane, k_off, qk_n, p.n_keys - 1 - tk * BN);
     else
       KTile::issue_at(gk1 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF, wave, lane, k_off, qk_n);
   };
-  auto load_k2 = [&](int tk, int buf) {
-    if (TAIL && (tk + 1) * BN > p.n_keys)
+  auto load_k2 = [&](int tk, int buf, auto tail) {
+    if (TAIL && decltype(tail)::value && (tk + 1) * BN > p.n_keys)
       KTile::issue_clamped(gk2 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF + C::K_TILE, wave, lane, k_off, qk_n, p.n_keys - 1 - tk * BN);
     else
       KTile::issue_at(gk2 + (size_t)tk * BN * qk_n, sKbuf + buf * C::K_BUF + C::K_TILE, wave, lane, k_off, qk_n);
   };
-  auto load_va = [&](int tv, int buf) {
-    if (TAIL && (tv + 1) * BN > p.n_keys)
+  auto load_va = [&](int tv, int buf, auto tail) {
+    if (TAIL && decltype(tail)::value && (tv + 1) * BN > p.n_keys)
       VTile::template issue_clamped<0, VH>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n, p.n_keys - 1 - tv * BN);
     else
       VTile::template issue_at<0, VH>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n);
   };
-  auto load_vb = [&](int tv, int buf) {
-    if (TAIL && (tv + 1) * BN > p.n_keys)
+  auto load_vb = [&](int tv, int buf, auto tail) {
+    if (TAIL && decltype(tail)::value && (tv + 1) * BN > p.n_keys)
       VTile::template issue_clamped<VH, VTile::PER>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n, p.n_keys - 1 - tv * BN);
     else
       VTile::template issue_at<VH, VTile::PER>(gv + (size_t)tv * BN * v_n, sVbuf + buf * C::V_TILE, wave, lane, v_off, v_n);
   };
+  constexpr std::true_type with_tail{};
+  constexpr std::false_type no_tail{};
 
   // Per-lane LDS byte addresses, computed once.  The XOR swizzle makes the address of a fragment a
   // different function of the lane for every 16-byte chunk column, so there is one register per chunk
@@ -220,9 +223,10 @@ void fwd_kernel(FwdParams p) {
   const bool head_half = (n_tiles & 2) != 0;
   const int b0 = head_half ? 2 : 0;
   // prologue: K tiles 0..2 and V tiles 0..1; scores of tile 0
-  load_k1(0, b0); load_k2(0, b0); load_va(0, b0); load_vb(0, b0);
-  load_k1(clampt(1), b0 + 1); load_k2(clampt(1), b0 + 1); load_va(clampt(1), b0 + 1); load_vb(clampt(1), b0 + 1);
-  load_k1(clampt(2), (b0 + 2) % 4); load_k2(clampt(2), (b0 + 2) % 4);
+  load_k1(0, b0, with_tail); load_k2(0, b0, with_tail); load_va(0, b0, with_tail); load_vb(0, b0, with_tail);
+  load_k1(clampt(1), b0 + 1, with_tail); load_k2(clampt(1), b0 + 1, with_tail);
+  load_va(clampt(1), b0 + 1, with_tail); load_vb(clampt(1), b0 + 1, with_tail);
+  load_k1(clampt(2), (b0 + 2) % 4, with_tail); load_k2(clampt(2), (b0 + 2) % 4, with_tail);
   wait_async_tiles();
   __syncthreads();
   f16v s_a[QS][NKT], s_b[QS][NKT];
@@ -238,7 +242,9 @@ void fwd_kernel(FwdParams p) {
   // POS = (t + b0) % NBUF is the ring position: K tile t+1 is read from buffer POS+1 and V tile t from
   // buffer POS; K tile t+3 goes to buffer POS+3 (tile t-1, consumed two iterations ago) and V tile t+2 to
   // buffer POS+2 (tile t-2, likewise), all modulo NBUF.
-  auto iteration = [&](int t, auto pos_tag, f16v (&s_cur)[QS][NKT], f16v (&s_nxt)[QS][NKT]) {
+  // `tail`: the iteration can meet tiles that reach past the last real key (their copies are clamped and, in
+  // the padded variant, their keys masked); iterations that cannot are compiled without those tests.
+  auto iteration = [&](int t, auto pos_tag, auto tail, f16v (&s_cur)[QS][NKT], f16v (&s_nxt)[QS][NKT]) {
     constexpr int POS = decltype(pos_tag)::value;
     constexpr int KR = (POS + 1) % 4, KP = (POS + 3) % 4, VR = POS, VP = (POS + 2) % 4;
     // Asynchronous prefetch straight into LDS, two iterations ahead: K tile t+3 and V tile t+2.
@@ -246,7 +252,7 @@ void fwd_kernel(FwdParams p) {
     // queue up behind each other at the memory pipeline.
     const int tk = clampt(t + 3);
     const int tv = clampt(t + 2);
-    load_k1(tk, KP);
+    load_k1(tk, KP, tail);
 
     // K fragments of the next tile are requested first; the row maxima of this tile are reduced
     // while they arrive.
@@ -267,7 +273,7 @@ void fwd_kernel(FwdParams p) {
       }
     }
 
-    if constexpr (PADDED) {
+    if constexpr (PADDED && decltype(tail)::value) {
       // only the last tiles hold padding keys
       if ((t + 1) * BN > p.n_keys) {
         const int rel = p.n_keys - 1 - t * BN - 4 * g;   // last real key minus the key index of register 0, tile 0
@@ -282,7 +288,7 @@ void fwd_kernel(FwdParams p) {
     // The score product of the next tile goes to the matrix unit first and runs under the row maxima and
     // the exponentials of this tile.  It starts from the running reference as it stands before this
     // tile's update; when the update moves the reference, the few results are corrected with it.
-    load_k2(tk, KP);
+    load_k2(tk, KP, tail);
     scores(ka, s_nxt);
 
     float mx[QS];
@@ -376,8 +382,8 @@ void fwd_kernel(FwdParams p) {
 #pragma unroll
     for (int i = 0; i < NPV; ++i) {
       const int kk = i / NOT, tt = i % NOT;
-      if (i == 0) load_va(tv, VP);
-      if (i == NPV / 2) load_vb(tv, VP);
+      if (i == 0) load_va(tv, VP, tail);
+      if (i == NPV / 2) load_vb(tv, VP, tail);
       if (i + PD < NPV) vfr[i + PD] = vt_frag(i + PD);
 #pragma unroll
       for (int qs = 0; qs < QS; ++qs) o[qs][tt] = mfma32(vfr[i], __builtin_bit_cast(h8, pw[qs][kk]), o[qs][tt]);
@@ -397,17 +403,25 @@ void fwd_kernel(FwdParams p) {
   // the tile count is even (N is a multiple of 128, tiles are at most 64 keys)
   int t = 0;
   if (head_half) {
-    iteration(0, std::integral_constant<int, 2>{}, s_a, s_b);
-    iteration(1, std::integral_constant<int, 3>{}, s_b, s_a);
+    iteration(0, std::integral_constant<int, 2>{}, with_tail, s_a, s_b);
+    iteration(1, std::integral_constant<int, 3>{}, with_tail, s_b, s_a);
     t = 2;
   }
+  auto turn = [&](int t, auto tail) {
+    iteration(t, std::integral_constant<int, 0>{}, tail, s_a, s_b);
+    iteration(t + 1, std::integral_constant<int, 1>{}, tail, s_b, s_a);
+    iteration(t + 2, std::integral_constant<int, 2>{}, tail, s_a, s_b);
+    iteration(t + 3, std::integral_constant<int, 3>{}, tail, s_b, s_a);
+  };
+  if constexpr (PADDED) {
+    // Padding concerns the last tiles only: an iteration copies K tile t+3, so the first one that can touch a
+    // tile with padding rows is number n_keys / BN - 3.  Whole turns in front of it run without the tests.
+    const int t_tail = p.n_keys / BN - 3;
 #pragma nounroll
-  for (; t < n_tiles; t += 4) {
-    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b);
-    iteration(t + 1, std::integral_constant<int, 1>{}, s_b, s_a);
-    iteration(t + 2, std::integral_constant<int, 2>{}, s_a, s_b);
-    iteration(t + 3, std::integral_constant<int, 3>{}, s_b, s_a);
+    for (; t + 4 <= t_tail; t += 4) turn(t, no_tail);
   }
+#pragma nounroll
+  for (; t < n_tiles; t += 4) turn(t, with_tail);
 
   wait_async_tiles();   // the staging blocks below reuse the tile memory the last prefetches write to
   __syncthreads();
