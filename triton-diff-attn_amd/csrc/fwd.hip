@@ -131,6 +131,7 @@ void fwd_kernel(FwdParams p) {
     m[qs] = 0.f; l[qs] = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) negm[qs][r] = 0.f;
+    asm volatile("" : "+v"(negm[qs]));   // sixteen registers of its own: the score products take it as their C operand as it is
   }
 
   using KTile = AsyncTile<BN, D, NW>;
@@ -330,6 +331,7 @@ void fwd_kernel(FwdParams p) {
           for (int r = 0; r < 16; ++r) { s_cur[qs][kt][r] -= d; s_nxt[qs][kt][r] -= d; }
 #pragma unroll
         for (int r = 0; r < 16; ++r) negm[qs][r] = -m[qs];
+        asm volatile("" : "+v"(negm[qs]));
       }
     }
 
