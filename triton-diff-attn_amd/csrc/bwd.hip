@@ -785,8 +785,8 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
 #pragma unroll
     for (int kv = 0; kv < NKV; ++kv) xf[kv] = *reinterpret_cast<const h8*>(rx + 16 * kv);
   }
-  const float nl1 = p.stat[0 * rows + qrow], nl2 = p.stat[1 * rows + qrow];
-  const float de1 = p.stat[2 * rows + qrow], de2 = p.stat[3 * rows + qrow];
+  const float nl1_ld = p.stat[0 * rows + qrow], nl2_ld = p.stat[1 * rows + qrow];
+  const float de1_ld = p.stat[2 * rows + qrow], de2_ld = p.stat[3 * rows + qrow];
 
   f16v dq1[NDT], dq2[NDT];
 #pragma unroll
@@ -831,6 +831,14 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   };
   fetch_all(0, 0);
   fetch_all((n_tiles > 1) ? 1 : 0, 1);
+  // dX and the row statistics are first used inside the loop, and the compiler waits for a load where it is first
+  // used.  It does not see the asynchronous tile copies, so its wait for "the newest loads" would in fact be a
+  // wait for every tile copy in flight, in every iteration.  Touching the registers here puts that wait in front
+  // of the loop, where the first tiles are waited for anyway.
+#pragma unroll
+  for (int kv = 0; kv < NKV; ++kv) asm volatile("" : "+v"(xf[kv]));
+  float nl1 = nl1_ld, nl2 = nl2_ld, de1 = de1_ld, de2 = de2_ld;
+  asm volatile("" : "+v"(nl1), "+v"(nl2), "+v"(de1), "+v"(de2));
   if (C::PAIR) wait_async_tiles();                  // tiles 0 and 1 are read before the next barrier
   else wait_async_tiles_except(loads_per_iter);     // tile 0 has landed, tile 1 may still be in flight
   __syncthreads();

@@ -202,16 +202,34 @@ void fwd_kernel(FwdParams p) {
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) ka[kt][ks] = lds_read_at<h8>(kb[ks], byte_off + kt * 32 * D * 2);
   };
-  auto scores = [&](const h8 (&ka)[NKT][NKS], f16v (&s)[QS][NKT]) {
+  // Score products number I0 .. I1-1 of a tile, counted in issue order: 32-key tile kt, k-step ks is number
+  // kt * NKS + ks.  The first product of a 32-key tile starts from the running reference.
+  auto scores_of = [&](const h8 (&ka)[NKT][NKS], f16v (&s)[QS][NKT], auto i0, auto i1) {
 #pragma unroll
-    for (int kt = 0; kt < NKT; ++kt)
+    for (int i = decltype(i0)::value; i < decltype(i1)::value; ++i) {
+      const int kt = i / NKS, ks = i % NKS;
 #pragma unroll
       for (int qs = 0; qs < QS; ++qs) {
-        s[qs][kt] = negm[qs];
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) s[qs][kt] = mfma32(ka[kt][ks], qf[qs][ks], s[qs][kt]);
+        if (ks == 0) s[qs][kt] = negm[qs];
+        s[qs][kt] = mfma32(ka[kt][ks], qf[qs][ks], s[qs][kt]);
       }
+    }
   };
+  constexpr int NSC = NKT * NKS;      // score products per tile and 32-row block
+  auto scores = [&](const h8 (&ka)[NKT][NKS], f16v (&s)[QS][NKT]) {
+    scores_of(ka, s, std::integral_constant<int, 0>{}, std::integral_constant<int, NSC>{});
+  };
+  // How many of the next tile's score products are issued ahead of the row maxima of this one; the rest follow
+  // the reference update and run under the first exponentials, which have no other matrix work beside them.
+  // The split is between 32-key tiles.  Measured against all of them ahead, inside one GPU call each: the
+  // first of two tiles ahead -2.5 % at D = 64 (0.442 -> 0.432 ms) and -1 % at D = 32; none ahead the same at
+  // D = 64 and +0.7 % at D = 128; a D = 128 tile is a single 32-key tile, and splitting it in the middle
+  // of its k-steps cost 1.5 %, so it stays whole and ahead.
+  constexpr int SC_EARLY = DROP ? NSC : ((NKT + 1) / 2) * NKS;
+  constexpr int KT_EARLY = (SC_EARLY + NKS - 1) / NKS;     // 32-key tiles whose first product is among them
+  constexpr std::integral_constant<int, 0> sc_first{};
+  constexpr std::integral_constant<int, SC_EARLY> sc_split{};
+  constexpr std::integral_constant<int, NSC> sc_end{};
 
   // loads this wave issues per iteration (one K1, one K2 and one V tile)
   const int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
@@ -290,7 +308,7 @@ void fwd_kernel(FwdParams p) {
     // the exponentials of this tile.  It starts from the running reference as it stands before this
     // tile's update; when the update moves the reference, the few results are corrected with it.
     load_k2(tk, KP, tail);
-    scores(ka, s_nxt);
+    scores_of(ka, s_nxt, sc_first, sc_split);
 
     float mx[QS];
 #pragma unroll
@@ -328,7 +346,10 @@ void fwd_kernel(FwdParams p) {
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) { s_cur[qs][kt][r] -= d; s_nxt[qs][kt][r] -= d; }
+          for (int r = 0; r < 16; ++r) {
+            s_cur[qs][kt][r] -= d;
+            if (kt < KT_EARLY) s_nxt[qs][kt][r] -= d;     // the later ones start from the new reference
+          }
 #pragma unroll
         for (int r = 0; r < 16; ++r) negm[qs][r] = -m[qs];
         asm volatile("" : "+v"(negm[qs]));
@@ -340,6 +361,23 @@ void fwd_kernel(FwdParams p) {
     // dropout: the mask arithmetic needs the registers of the K fragments, so the score product is
     // issued in full before the exponentials instead of between them
     if constexpr (DROP) __builtin_amdgcn_sched_barrier(0);
+
+    // V^T fragments are requested PD products ahead of the product that uses them (measured: 2 and
+    // 3 are 1.3 % faster than the single product the compiler picks by itself, 5 and 7 are not); the
+    // first ones here, so that they arrive under the exponentials
+    constexpr int NPV = NKK * NOT;
+    constexpr int PD = DROP ? 1 : 3;           // dropout: registers are short
+    auto vt_frag = [&](int i) {
+      const int kk = i / NOT, tt = i % NOT;
+      const int off = VR * C::VBUF_BYTES + 16 * kk * DV * 2;
+      return join(lds_read_tr_at(vtr[tt][0], off), lds_read_tr_at(vtr[tt][1], off));
+    };
+    h8 vfr[NPV];
+    if constexpr (!DROP) {
+#pragma unroll
+      for (int i = 0; i < PD && i < NPV; ++i) vfr[i] = vt_frag(i);
+    }
+    scores_of(ka, s_nxt, sc_split, sc_end);
 
     // P^T as B operands: pb[kk] covers keys 16kk..16kk+15 (accumulator order).  Built from the packed
     // pairs as 32-bit words, so that each pair is converted once, for the row sum and the operand alike.
@@ -369,18 +407,10 @@ void fwd_kernel(FwdParams p) {
       l[qs] += rs;
     }
 
-    // V^T fragments are requested PD products ahead of the product that uses them (measured: 2 and
-    // 3 are 1.3 % faster than the single product the compiler picks by itself, 5 and 7 are not)
-    constexpr int NPV = NKK * NOT;
-    constexpr int PD = DROP ? 1 : 3;           // dropout: registers are short
-    auto vt_frag = [&](int i) {
-      const int kk = i / NOT, tt = i % NOT;
-      const int off = VR * C::VBUF_BYTES + 16 * kk * DV * 2;
-      return join(lds_read_tr_at(vtr[tt][0], off), lds_read_tr_at(vtr[tt][1], off));
-    };
-    h8 vfr[NPV];
+    if constexpr (DROP) {
 #pragma unroll
-    for (int i = 0; i < PD && i < NPV; ++i) vfr[i] = vt_frag(i);
+      for (int i = 0; i < PD && i < NPV; ++i) vfr[i] = vt_frag(i);
+    }
 #pragma unroll
     for (int i = 0; i < NPV; ++i) {
       const int kk = i / NOT, tt = i % NOT;
