@@ -707,14 +707,17 @@ struct DqCfg {
   static constexpr int K_TILE = BN * D;        // halfs (swizzled, unpadded)
   static constexpr int V_TILE = BN * DV;
   static constexpr int STAGE = 2 * K_TILE + V_TILE;
-  // Ring depth.  Tiles are fetched two iterations ahead, which takes three buffers and a barrier per tile.
-  // With four buffers the workgroup has to meet only every second tile (a tile's buffer is refilled two tiles
-  // after it was read, which is always past one barrier), so the two waves of a SIMD, which leave a barrier in
-  // step, have twice as long to drift apart and overlap one's matrix products with the other's element-wise
-  // work.  Measured in one GPU call against the three-buffer ring: 3.6 % faster at D = 128, 0.8 % at D = 32,
-  // 2 % slower at D = 64, which therefore keeps three buffers.
+  // A ring of four buffers whose position is a compile-time constant in every iteration (the loop body is one
+  // turn of the ring), laid out by tile kind so that an instruction's immediate offset reaches every buffer.
+  // Tiles are fetched two iterations ahead.  With a barrier per tile three buffers would do; four let the
+  // workgroup meet every second tile only (a tile's buffer is refilled two tiles after it was read, which is
+  // always past one barrier), so the two waves of a SIMD, which leave a barrier in step, have twice as long to
+  // drift apart and overlap one's matrix products with the other's element-wise work.  Measured in one GPU call
+  // against a barrier per tile: 3.6 % faster at D = 128, 0.8 % at D = 32, 2 % slower at D = 64.
   static constexpr bool PAIR = (D != 64);      // a barrier every second tile
-  static constexpr int NBUF = PAIR ? 4 : 3;
+  static constexpr int NBUF = 4;
+  static constexpr int KBUF_BYTES = 2 * K_TILE * 2, VBUF_BYTES = V_TILE * 2, VBASE_BYTES = NBUF * KBUF_BYTES;
+  static_assert(NBUF * KBUF_BYTES <= 65536 && NBUF * VBUF_BYTES <= 65536, "immediate offsets reach every buffer");
 };
 
 // dQ_t = s * dS_t K_t for one block of query rows.  Every product is formed transposed,
@@ -802,14 +805,12 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   const unsigned k_off = KTile::lane_off(wave, lane, qk_n), v_off = VTile::lane_off(wave, lane, v_n);
   // causal: keys beyond the last row of the workgroup are never visited
   // padding: tiles that hold no real key are not visited either
-  const int n_tiles = CAUSAL ? (qt + 1) * (BM / BN) : PADDED ? (p.n_keys + BN - 1) / BN : p.N / BN;
+  // (an even count in every variant: with padding, a last tile without a real key may be visited; its keys are masked)
+  const int n_tiles = CAUSAL ? (qt + 1) * (BM / BN) : PADDED ? (((p.n_keys + BN - 1) / BN + 1) & ~1) : p.N / BN;
   constexpr int VH = (VTile::PER + 1) / 2;
 
-  int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
-  // At D = 128 the count is hidden from the compiler, although it is the same for every wave: as a constant it
-  // merges the end of an iteration into one block with the next iteration's fragment reads, and the schedule it
-  // then picks was measured 13 % slower (1.94 against 2.19 ms at B2 H32 N4096, same GPU call).
-  if (D == 128) asm volatile("" : "+s"(loads_per_iter));
+  // loads a wave issues per iteration (one K1, one K2 and one V tile)
+  const int loads_per_iter = 2 * KTile::count(wave) + VTile::count(wave);
   // with padding, the tiles that reach past the last real key are copied with their row index clamped to it
   auto copy_k = [&](const half_t* gk, int t, half_t* dst) {
     if (TAIL && (t + 1) * BN > p.n_keys) KTile::issue_clamped(gk + (size_t)t * BN * qk_n, dst, wave, lane, k_off, qk_n, p.n_keys - 1 - t * BN);
@@ -823,14 +824,21 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   constexpr std::integral_constant<int, 0> v_begin{};
   constexpr std::integral_constant<int, VH> v_mid{};
   constexpr std::integral_constant<int, VTile::PER> v_end{};
+  // tile memory by kind: K1 and K2 of buffer b, then the V tiles
+  auto k_buf = [&](int b) { return smem + b * (C::KBUF_BYTES / 2); };
+  auto v_buf = [&](int b) { return smem + C::VBASE_BYTES / 2 + b * C::V_TILE; };
   auto fetch_all = [&](int t, int buf) {
-    half_t* b = smem + buf * C::STAGE;
-    copy_k(gk1, t, b);
-    copy_k(gk2, t, b + C::K_TILE);
-    copy_v(t, b + 2 * C::K_TILE, v_begin, v_end);
+    copy_k(gk1, t, k_buf(buf));
+    copy_k(gk2, t, k_buf(buf) + C::K_TILE);
+    copy_v(t, v_buf(buf), v_begin, v_end);
   };
-  fetch_all(0, 0);
-  fetch_all((n_tiles > 1) ? 1 : 0, 1);
+  // The loop runs whole turns of the ring (NBUF iterations); the tile count is even, so when it is not a
+  // multiple of four, half a turn comes first and tile 0 goes into buffer 2: tile t is in buffer (t + b0) % NBUF.
+  static_assert(C::NBUF == 4, "the loop is unrolled over a ring of four");
+  const bool head_half = (n_tiles & 2) != 0;
+  const int b0 = head_half ? 2 : 0;
+  fetch_all(0, b0);
+  fetch_all((n_tiles > 1) ? 1 : 0, b0 + 1);
   // dX and the row statistics are first used inside the loop, and the compiler waits for a load where it is first
   // used.  It does not see the asynchronous tile copies, so its wait for "the newest loads" would in fact be a
   // wait for every tile copy in flight, in every iteration.  Touching the registers here puts that wait in front
@@ -842,22 +850,42 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   if (C::PAIR) wait_async_tiles();                  // tiles 0 and 1 are read before the next barrier
   else wait_async_tiles_except(loads_per_iter);     // tile 0 has landed, tile 1 may still be in flight
   __syncthreads();
-  int bcur = 0, bnext = 2;   // buffer of tile t, buffer that receives tile t+2
 
+  // Per-lane LDS byte addresses, computed once.  The XOR swizzle makes the address of a fragment a different
+  // function of the lane for every 16-byte chunk column, so there is one register per chunk column a lane
+  // reads; the ring buffer, K1 or K2, the 32-key sub-tile and the k-step of 16 keys are multiples of 16 rows,
+  // which the swizzle does not see, and travel in the instructions' immediate offsets.
   const int tr_row = 4 * g + ((lane & 15) >> 2);
   const int tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const unsigned lds0 = (unsigned)(unsigned long)((DA_LDS char*)smem);
+  unsigned kfr[NKS], vfr[NKV], ktr[NDT][2];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) kfr[ks] = lds0 + 2u * (unsigned)swz_off<D>(j, 16 * ks + 8 * g);
+#pragma unroll
+  for (int kv = 0; kv < NKV; ++kv) vfr[kv] = lds0 + C::VBASE_BYTES + 2u * (unsigned)swz_off<DV>(j, 16 * kv + 8 * g);
+#pragma unroll
+  for (int tt = 0; tt < NDT; ++tt)
+#pragma unroll
+    for (int e = 0; e < 2; ++e) ktr[tt][e] = lds0 + 2u * (unsigned)swz_off<D>(tr_row + 8 * e, 32 * tt + tr_col);
+  // kept as they are: the compiler neither folds constants into them nor recomputes them in the loop
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) asm volatile("" : "+v"(kfr[ks]));
+#pragma unroll
+  for (int kv = 0; kv < NKV; ++kv) asm volatile("" : "+v"(vfr[kv]));
+#pragma unroll
+  for (int tt = 0; tt < NDT; ++tt) asm volatile("" : "+v"(ktr[tt][0]), "+v"(ktr[tt][1]));
 
-  for (int t = 0; t < n_tiles; ++t) {
-    const half_t* sK1 = smem + bcur * C::STAGE;
-    const half_t* sK2 = sK1 + C::K_TILE;
-    const half_t* sV = sK1 + 2 * C::K_TILE;
-    half_t* nb = smem + bnext * C::STAGE;            // held a tile that every wave has finished reading
+  // One iteration: tile t, in the buffer at ring position POS; tile t+2 is requested into the buffer two
+  // positions on, which held a tile that every wave has finished reading.
+  auto iteration = [&](int t, auto pos_tag) {
+    constexpr int POS = decltype(pos_tag)::value;
+    constexpr int KCUR = POS * C::KBUF_BYTES, VCUR = POS * C::VBUF_BYTES, BNXT = (POS + 2) % C::NBUF;
     const int tn = (t + 2 < n_tiles) ? t + 2 : n_tiles - 1;   // past the end: harmless re-reads
-    copy_k(gk1, tn, nb);
+    copy_k(gk1, tn, k_buf(BNXT));
 
 #pragma unroll
     for (int ksub = 0; ksub < BN / 32; ++ksub) {
-      if (ksub == 0) copy_k(gk2, tn, nb + C::K_TILE);
+      if (ksub == 0) copy_k(gk2, tn, k_buf(BNXT) + C::K_TILE);
       // transposed tiles [32 keys x 32 queries]: this lane's column is its query
       f16v s1, s2, dp;
 #pragma unroll
@@ -866,12 +894,11 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       h8 ak1[NKS], ak2[NKS], av[NKV];
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
-        ak1[ks] = *reinterpret_cast<const h8*>(sK1 + swz_off<D>(ksub * 32 + j, 16 * ks + 8 * g));
-        ak2[ks] = *reinterpret_cast<const h8*>(sK2 + swz_off<D>(ksub * 32 + j, 16 * ks + 8 * g));
+        ak1[ks] = lds_read_at<h8>(kfr[ks], KCUR + ksub * 32 * D * 2);
+        ak2[ks] = lds_read_at<h8>(kfr[ks], KCUR + C::K_TILE * 2 + ksub * 32 * D * 2);
       }
 #pragma unroll
-      for (int kv = 0; kv < NKV; ++kv)
-        av[kv] = *reinterpret_cast<const h8*>(sV + swz_off<DV>(ksub * 32 + j, 16 * kv + 8 * g));
+      for (int kv = 0; kv < NKV; ++kv) av[kv] = lds_read_at<h8>(vfr[kv], VCUR + ksub * 32 * DV * 2);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
@@ -880,9 +907,9 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       }
 #pragma unroll
       for (int kv = 0; kv < NKV; ++kv) dp = mfma32(av[kv], xf[kv], dp);
-      if (ksub == 0) copy_v(tn, nb + 2 * C::K_TILE, v_begin, v_mid);
+      if (ksub == 0) copy_v(tn, v_buf(BNXT), v_begin, v_mid);
       // with a barrier every second tile all of a tile's copies go out early: they have to land by the next barrier
-      if (ksub == (C::PAIR ? 0 : BN / 32 - 1)) copy_v(tn, nb + 2 * C::K_TILE, v_mid, v_end);
+      if (ksub == (C::PAIR ? 0 : BN / 32 - 1)) copy_v(tn, v_buf(BNXT), v_mid, v_end);
       if constexpr (CAUSAL) {
         // only the last sub-tiles of a wave's loop reach past its first row: mask key > query there
         const int wrow0 = qt * BM + wave * 32;
@@ -911,11 +938,9 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       // fragment in front of its product instead.)
       h8 tk1[2][NDT], tk2[2][NDT];
       auto read_tk = [&](int kk, int tt) {
-        const int rbase = ksub * 32 + 16 * kk + tr_row;
-        tk1[kk][tt] = join(lds_read_tr(sK1 + swz_off<D>(rbase, 32 * tt + tr_col)),
-                           lds_read_tr(sK1 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
-        tk2[kk][tt] = join(lds_read_tr(sK2 + swz_off<D>(rbase, 32 * tt + tr_col)),
-                           lds_read_tr(sK2 + swz_off<D>(rbase + 8, 32 * tt + tr_col)));
+        const int off = KCUR + (ksub * 32 + 16 * kk) * D * 2;
+        tk1[kk][tt] = join(lds_read_tr_at(ktr[tt][0], off), lds_read_tr_at(ktr[tt][1], off));
+        tk2[kk][tt] = join(lds_read_tr_at(ktr[tt][0], off + C::K_TILE * 2), lds_read_tr_at(ktr[tt][1], off + C::K_TILE * 2));
       };
       // (At D = 128 the masked variants, which also carry the row clamping of padded sequences, are short of
       // registers in the same way.)
@@ -968,7 +993,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
     if constexpr (C::PAIR) {
       // Every second tile the workgroup meets: the copies of the next two tiles (requested during the last
       // two) have landed for everybody, and the buffers of the last two tiles may be refilled.
-      if (t & 1) {
+      if constexpr (POS & 1) {
         wait_async_tiles();
         __syncthreads();
       }
@@ -977,8 +1002,20 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       wait_async_tiles_except(loads_per_iter);
       __syncthreads();
     }
-    bcur = (bcur == C::NBUF - 1) ? 0 : bcur + 1;
-    bnext = (bnext == C::NBUF - 1) ? 0 : bnext + 1;
+  };
+
+  int t = 0;
+  if (head_half) {
+    iteration(0, std::integral_constant<int, 2>{});
+    iteration(1, std::integral_constant<int, 3>{});
+    t = 2;
+  }
+#pragma nounroll
+  for (; t < n_tiles; t += 4) {
+    iteration(t, std::integral_constant<int, 0>{});
+    iteration(t + 1, std::integral_constant<int, 1>{});
+    iteration(t + 2, std::integral_constant<int, 2>{});
+    iteration(t + 3, std::integral_constant<int, 3>{});
   }
   wait_async_tiles();
   __syncthreads();      // the tile memory is reused below; other waves may still have been reading it
