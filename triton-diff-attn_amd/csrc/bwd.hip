@@ -875,6 +875,22 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
 #pragma unroll
   for (int tt = 0; tt < NDT; ++tt) asm volatile("" : "+v"(ktr[tt][0]), "+v"(ktr[tt][1]));
 
+  // Where registers allow, a row statistic that is added to every element of a product is the product's
+  // initial accumulator value instead: sixteen registers that hold it, for sixteen additions less per sub-tile.
+#ifndef DQ_FOLD_DP
+#define DQ_FOLD_DP (!DROP && (D == 32 || (D == 64 && MASK == 0)))
+#endif
+#ifndef DQ_FOLD_S
+#define DQ_FOLD_S (D == 32)
+#endif
+  constexpr bool kFoldDP = DQ_FOLD_DP;     // dP starts from -delta1 (not with dropout, which masks dP first)
+  constexpr bool kFoldS = DQ_FOLD_S;       // S1, S2 start from the negated logsumexp
+  f16v de1v, nl1v, nl2v;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { de1v[r] = kFoldDP ? de1 : 0.f; nl1v[r] = kFoldS ? nl1 : 0.f; nl2v[r] = kFoldS ? nl2 : 0.f; }
+  if constexpr (kFoldDP) asm volatile("" : "+v"(de1v));
+  if constexpr (kFoldS) asm volatile("" : "+v"(nl1v), "+v"(nl2v));
+
   // One iteration: tile t, in the buffer at ring position POS; tile t+2 is requested into the buffer two
   // positions on, which held a tile that every wave has finished reading.
   auto iteration = [&](int t, auto pos_tag) {
@@ -887,9 +903,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
     for (int ksub = 0; ksub < BN / 32; ++ksub) {
       if (ksub == 0) copy_k(gk2, tn, k_buf(BNXT) + C::K_TILE);
       // transposed tiles [32 keys x 32 queries]: this lane's column is its query
-      f16v s1, s2, dp;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { s1[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
+      f16v s1 = nl1v, s2 = nl2v, dp = de1v;       // zero, or the folded statistic
       // all fragments of the three score products are requested before the first product is issued
       h8 ak1[NKS], ak2[NKS], av[NKV];
 #pragma unroll
@@ -956,8 +970,8 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       unsigned w1 = 0, w2 = 0;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float p1 = fast_exp2(s1[r] + nl1);
-        const float p2 = fast_exp2(s2[r] + nl2);
+        const float p1 = fast_exp2(kFoldS ? s1[r] : s1[r] + nl1);
+        const float p2 = fast_exp2(kFoldS ? s2[r] : s2[r] + nl2);
         if constexpr (DROP) {
           // register r holds key kq + 8*(r/4) + (r%4) of this lane's query; registers r, r+1 (r even)
           // share the hash words of their 2x2 block
@@ -975,7 +989,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
         } else {
           // in fp32 up to the rounding of dS itself: dP - delta alone may exceed the 16-bit range when the
           // upstream gradient carries a loss scale, while its product with the probability does not
-          const float dpc = dp[r] + de1;                  // statistic 2 is -delta1
+          const float dpc = kFoldDP ? dp[r] : dp[r] + de1;                  // statistic 2 is -delta1
           b1[r / 8][r % 8] = (half_t)(p1 * dpc);
           b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dpc, de2));   // statistic 3 is -(lambda*delta1 + delta2)
         }
