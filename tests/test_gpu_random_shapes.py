@@ -21,7 +21,9 @@ def draw(seed):
         bf16=rnd.random() < 0.3, lambda_init=rnd.choice([0.2, 0.5, 0.8]), seed=seed)
 
 
-@pytest.mark.parametrize("seed", range(24))
+# seed 247: bf16, causal, lambda 0.97 -- early rows in which the two streams nearly cancel, where a lambda-combine
+# formed from a 16-bit rounded stream is amplified by the norm past the tolerance (the combine is in fp32)
+@pytest.mark.parametrize("seed", list(range(24)) + [247])
 def test_random_problem_matches_oracle(seed):
     from layers import MultiheadDiffAttnKernel
 
@@ -59,7 +61,8 @@ def test_random_problem_matches_oracle(seed):
     assert (lam_dev.grad.float().cpu() - ref[6]).abs().max().item() <= (3 * g_tol) * denom
 
 
-@pytest.mark.parametrize("seed", range(100, 112))
+# seed 112: causal with dropout at D = 128 -- a first row whose single weight is kept in both streams cancels to (1 - lambda) v
+@pytest.mark.parametrize("seed", range(100, 113))
 def test_random_problem_with_dropout_and_strided_tensors(seed):
     """As above, with dropout drawn in and, for every other seed, the tensors living in [B,N,H,C] buffers."""
     from layers import MultiheadDiffAttnKernel

@@ -43,7 +43,11 @@ struct FwdCfg {
   static constexpr int KBUF_BYTES = K_BUF * 2, VBUF_BYTES = V_TILE * 2, VBASE_BYTES = NBUF * KBUF_BYTES;
   static_assert(NBUF * KBUF_BYTES <= 65536 && NBUF * VBUF_BYTES <= 65536, "immediate offsets reach every buffer");
   static constexpr int TILES = NBUF * (K_BUF + V_TILE);
-  static constexpr int XCHG = NW * 32 * (DV + 8);            // halfs needed by the epilogue staging blocks
+  // halfs needed by the epilogue: per pair of waves (stream 1, stream 2 of the same 32 rows) an fp32 exchange
+  // block of 32 x DV values, which the stream-1 wave reuses for its staged rows, and the staging block
+  // (32 rows of DV + 8 halfs) of the stream-2 wave
+  static constexpr int XCH_BLOCK = 64 * DV;
+  static constexpr int XCHG = (NW / 2) * (XCH_BLOCK + 32 * (DV + 8));
   static constexpr int SMEM = (TILES > XCHG) ? TILES : XCHG;
 };
 
@@ -458,14 +462,20 @@ void fwd_kernel(FwdParams p) {
   wait_async_tiles();   // the staging blocks below reuse the tile memory the last prefetches write to
   __syncthreads();
   // ---- epilogue ----------------------------------------------------------------------------
-  // Every row quantity is per query = per lane pair (l, l^32).  Each wave owns a staging block of
+  // Every row quantity is per query = per lane pair (l, l^32).  Each wave has a staging block of
   // 32 rows x DV halfs in the now idle tile memory (row stride DV+8 halfs).  Results are written
   // there in accumulator layout (8 bytes per lane) and read back row by row, so that the global
   // stores are whole 16-byte chunks of consecutive rows.  The stream-2 waves stage softmax(S2)V
-  // rounded to fp16 -- the tensor saved for backward -- and the stream-1 wave that owns the same
-  // rows reads it from there for the lambda-combine.
+  // rounded to 16 bits -- the tensor saved for backward -- and also hand it, unrounded, to the stream-1
+  // wave that owns the same rows: the lambda-combine is formed in fp32, as in the reference
+  // (src/kernel.py:191-194), so that rows in which the two streams nearly cancel (lambda near 1, similar
+  // attention maps) do not see the rounding error of one stream amplified by the norm.  The two waves
+  // hold a row's values in the same lanes and registers, so the exchange is lane to lane.
   constexpr int SROW = DV + 8;
-  half_t* const stg_own = smem + (size_t)wave * 32 * SROW;
+  float* const xch = reinterpret_cast<float*>(smem + (size_t)qw * C::XCH_BLOCK);
+  // stream 1 stages its rows in its pair's exchange block, which only this wave reads, after reading it
+  half_t* const stg_own = st ? smem + (size_t)(NW / 2) * C::XCH_BLOCK + (size_t)qw * 32 * SROW
+                             : smem + (size_t)qw * C::XCH_BLOCK;
   auto stage_rows = [&](int qs, const f16v (&val)[NOT], float scale) {
 #pragma unroll
     for (int tt = 0; tt < NOT; ++tt)
@@ -500,22 +510,32 @@ void fwd_kernel(FwdParams p) {
     float* lse = st ? p.lse2 : p.lse1;
     if (g == 0 && lse) lse[row] = (m[0] + __builtin_log2f(lsum)) * kLn2;
   }
-  if (st == 1) stage_rows(0, o[0], inv);
+  if (st == 1) {
+    stage_rows(0, o[0], inv);
+#pragma unroll
+    for (int tt = 0; tt < NOT; ++tt)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        f4v u;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) u[e] = o[0][tt][4 * r4 + e] * inv;
+        *reinterpret_cast<f4v*>(xch + ((tt * 4 + r4) * 64 + lane) * 4) = u;
+      }
+  }
   __syncthreads();
   if (st == 1) {
     if (p.u2) store_rows(p.u2 + wave_row0 * DV, DV, 32);
   } else {
     const float lam = da_abi::lambda_of_unit(p, bh);
-    const half_t* stg_u2 = smem + (size_t)(wave + NW / 2) * 32 * SROW;
     float ss = 0.f;
 #pragma unroll
     for (int tt = 0; tt < NOT; ++tt)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
-        const h4 u = *reinterpret_cast<const h4*>(stg_u2 + j * SROW + 32 * tt + 8 * r4 + 4 * g);
+        const f4v u = *reinterpret_cast<const f4v*>(xch + ((tt * 4 + r4) * 64 + lane) * 4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float x = o[0][tt][4 * r4 + e] * inv - lam * (float)u[e];
+          const float x = o[0][tt][4 * r4 + e] * inv - lam * u[e];
           o[0][tt][4 * r4 + e] = x;
           ss += x * x;
         }
