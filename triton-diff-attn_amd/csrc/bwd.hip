@@ -407,7 +407,7 @@ __global__ __launch_bounds__((DkvCfg<D, NWAVES>::NT)) __attribute__((amdgpu_wave
   // Element-wise work of accumulator register r (query row 8*(r/4) + 4g + (r%4)), split in three
   // stages that are issued one product apart, so that no VALU instruction waits on the one
   // before it: (1) exponentials, (2) products, (3) fp16 packing of a pair of rows.
-  struct RowTmp { float p1[16], p2[16], u[16], ds1[16], ds2[16], pc[16], a1[16], k1[16], k2[16]; unsigned w1, w2; };
+  struct RowTmp { float p1[16], p2[16], u[16], ds1[16], ds2[16], pc[16], a1[16], k1[16], k2[16]; unsigned w1, w2, w1b, w2b; };
   // `rel` (masked steps only) = key index minus the query index of register 0 of the sub-tile:
   // register r holds query 8*(r/4) + (r%4) relative to that, and a query before its key sees nothing
   auto ew1 = [&](int r, const f4v& st3, const f4v& st2, const Scores& in, RowTmp& t, auto masked_tag, int rel, int qbase) {
@@ -420,12 +420,15 @@ __global__ __launch_bounds__((DkvCfg<D, NWAVES>::NT)) __attribute__((amdgpu_wave
       // register r holds query qbase + 8*(r/4) + (r%4) of this lane's key; registers r, r+1 (r even)
       // share the hash words of their 2x2 block, one word per softmax stream
       const unsigned query = (unsigned)(qbase + 8 * (r / 4) + (r % 4));
-      if ((r & 1) == 0) {
-        t.w1 = dropout_word(dkey1, (unsigned)p.N / 2, query >> 1, (unsigned)key >> 1);
-        t.w2 = dropout_word(dkey2, (unsigned)p.N / 2, query >> 1, (unsigned)key >> 1);
+      // the blocks of registers r..r+1 and r+2..r+3 (r a multiple of 4) are neighbours, hashed one by each
+      // lane of a key pair
+      if ((r & 3) == 0) {
+        const unsigned odd = (unsigned)key & 1u;
+        dropout_words_shared(dropout_word(dkey1, (unsigned)p.N / 2, (query >> 1) + odd, (unsigned)key >> 1), odd, t.w1, t.w1b);
+        dropout_words_shared(dropout_word(dkey2, (unsigned)p.N / 2, (query >> 1) + odd, (unsigned)key >> 1), odd, t.w2, t.w2b);
       }
-      const bool keep1 = dropout_keep(t.w1, query, (unsigned)key, p.drop.threshold);
-      const bool keep2 = dropout_keep(t.w2, query, (unsigned)key, p.drop.threshold);
+      const bool keep1 = dropout_keep((r & 2) ? t.w1b : t.w1, query, (unsigned)key, p.drop.threshold);
+      const bool keep2 = dropout_keep((r & 2) ? t.w2b : t.w2, query, (unsigned)key, p.drop.threshold);
       t.k1[r] = keep1 ? t.p1[r] : 0.f;
       t.k2[r] = keep2 ? t.p2[r] : 0.f;
       if constexpr (DO_K) {
@@ -967,7 +970,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
       }
       __builtin_amdgcn_sched_barrier(0);
       h8 b1[2], b2[2];
-      unsigned w1 = 0, w2 = 0;
+      unsigned w1 = 0, w2 = 0, w1b = 0, w2b = 0;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float p1 = fast_exp2(kFoldS ? s1[r] : s1[r] + nl1);
@@ -977,13 +980,15 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
           // share the hash words of their 2x2 block
           const unsigned query = (unsigned)(qt * BM + wave * 32 + j);
           const unsigned kq = (unsigned)(t * BN + ksub * 32 + 4 * g + 8 * (r / 4) + (r % 4));
-          if ((r & 1) == 0) {
-            w1 = dropout_word(dkey1, (unsigned)p.N / 2, query >> 1, kq >> 1);
-            w2 = dropout_word(dkey2, (unsigned)p.N / 2, query >> 1, kq >> 1);
+          // the blocks of registers r..r+1 and r+2..r+3 (r a multiple of 4) are neighbours, hashed one by each
+          // lane of a query pair
+          if ((r & 3) == 0) {
+            dropout_words_shared(dropout_word(dkey1, (unsigned)p.N / 2, query >> 1, (kq >> 1) + (query & 1)), query & 1, w1, w1b);
+            dropout_words_shared(dropout_word(dkey2, (unsigned)p.N / 2, query >> 1, (kq >> 1) + (query & 1)), query & 1, w2, w2b);
           }
           const float dpk = p.drop.keep_scale * dp[r];
-          const float d1 = dropout_keep(w1, query, kq, p.drop.threshold) ? dpk : 0.f;
-          const float d2 = dropout_keep(w2, query, kq, p.drop.threshold) ? dpk : 0.f;
+          const float d1 = dropout_keep((r & 2) ? w1b : w1, query, kq, p.drop.threshold) ? dpk : 0.f;
+          const float d2 = dropout_keep((r & 2) ? w2b : w2, query, kq, p.drop.threshold) ? dpk : 0.f;
           b1[r / 8][r % 8] = (half_t)(p1 * (d1 + de1));                                             // c m1 dP - delta1
           b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, d2, __builtin_fmaf(-lam, de1, de2)));   // -lambda c m2 dP - delta2
         } else {

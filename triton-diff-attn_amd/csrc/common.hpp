@@ -316,6 +316,15 @@ __device__ __forceinline__ unsigned dropout_word(const DropoutKey& key, unsigned
   h ^= h >> 16;
   return h;
 }
+// The word of a 2x2 block serves two lanes: the kernels hold the block's two queries (or its two keys) in lanes
+// l and l^1.  Of two neighbouring blocks each lane of the pair hashes one -- the even lane the first, the odd
+// lane the second (`mine`) -- and takes the other from its neighbour, which halves the hash work.
+// Every lane of the wave must be active.
+__device__ __forceinline__ void dropout_words_shared(unsigned mine, bool odd_lane, unsigned& first, unsigned& second) {
+  const unsigned other = (unsigned)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1 /* quad_perm 1,0,3,2 */, 0xF, 0xF, true);
+  first = odd_lane ? other : mine;
+  second = odd_lane ? mine : other;
+}
 // keep decision of pair (q, k) from the word of its 2x2 block
 __device__ __forceinline__ bool dropout_keep(unsigned word, unsigned q, unsigned k, unsigned threshold) {
   return ((word >> (8 * (2 * (q & 1) + (k & 1)))) & 0xffu) >= threshold;

@@ -389,6 +389,7 @@ void fwd_kernel(FwdParams p) {
 #pragma unroll
     for (int qs = 0; qs < QS; ++qs) {
       float rs = 0.f;
+      unsigned word_a = 0, word_b = 0;     // dropout: hash words of two neighbouring 2x2 blocks
 #pragma unroll
       for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
@@ -399,10 +400,14 @@ void fwd_kernel(FwdParams p) {
           rs = add_pair(e2, rs);   // row sum of the rounded probabilities
           unsigned w2 = __builtin_bit_cast(unsigned, e2);
           if constexpr (DROP) {
-            // registers r, r+1 hold the keys key, key+1 (key even) of this lane's query
+            // registers r, r+1 hold the keys key, key+1 (key even) of this lane's query; the blocks of registers
+            // r..r+1 and r+2..r+3 (r a multiple of 4) are neighbours, hashed one by each lane of a query pair
             const unsigned query = (unsigned)(qrow0 + 32 * qs);
             const unsigned key = (unsigned)(t * BN + kt * 32 + 8 * (r / 4) + 4 * g + (r % 4));
-            const unsigned word = dropout_word(dkey, (unsigned)p.N / 2, query >> 1, key >> 1);
+            if (r % 4 == 0)
+              dropout_words_shared(dropout_word(dkey, (unsigned)p.N / 2, query >> 1, (key >> 1) + (query & 1)), query & 1,
+                                   word_a, word_b);
+            const unsigned word = (r % 4 == 0) ? word_a : word_b;
             w2 &= (dropout_keep(word, query, key, p.drop.threshold) ? 0x0000ffffu : 0u) |
                   (dropout_keep(word, query, key + 1, p.drop.threshold) ? 0xffff0000u : 0u);
           }
