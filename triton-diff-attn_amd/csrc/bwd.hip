@@ -353,7 +353,9 @@ __global__ __launch_bounds__((DkvCfg<D, NWAVES>::NT)) __attribute__((amdgpu_wave
   constexpr int NPROD = 2 * NKS + (DO_K ? NKV : 0);   // score products per sub-tile (dP is needed for dK only)
   // the D = 128 instantiations with dropout are short of registers: they request one fragment ahead
   constexpr bool kShort = DROP && D == 128;
-  constexpr int DEPTH = kShort ? 1 : 3;        // A fragments requested ahead of their product
+  // A fragments requested ahead of their product (measured in one GPU call: 4 is 1 % faster than 3 at D = 64 and
+  // D = 128 and the same at D = 32; 5 and 6 spill in some instantiations and are not faster)
+  constexpr int DEPTH = kShort ? 1 : 4;
 
   // Product k of a sub-tile: even k is k-step k/2 of dP, odd k alternates k-steps of S1 and S2, so
   // the three accumulation chains advance together; without dP (MODE 1) S1 and S2 alternate.
@@ -521,7 +523,7 @@ __global__ __launch_bounds__((DkvCfg<D, NWAVES>::NT)) __attribute__((amdgpu_wave
   // of the step and read during the second, its upper half is written during the second half and
   // read during the first half of the next step.
   static_assert(NPROD % 16 == 0 || 16 % NPROD == 0, "rows are spread evenly over the products");
-  constexpr int AHEAD = kShort ? 1 : 3;        // B fragments requested ahead of their product
+  constexpr int AHEAD = kShort ? 1 : 3;        // B fragments requested ahead of their product (4: no faster)
   auto fused = [&](int bufn, int qsn, Scores& s_nxt, int bufc, int qsc, const Scores& s_cur, Packed& pk,
                    int bufp, int qsp, int tile_next, auto buf_next_tag, auto fetch_tag, auto masked_tag, int rel, int qbase) {
     constexpr int buf_next = decltype(buf_next_tag)::value;
