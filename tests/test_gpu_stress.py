@@ -88,3 +88,31 @@ def test_lambda_gradient_under_a_loss_scale(D):
             assert rel_to_max(g.float().cpu() / scale, r) <= GRAD_RTOL, name
     assert abs(got[torch.float32] - want) <= GRAD_RTOL * abs(want)
     assert got[torch.float16] == float("inf") * (1 if want > 0 else -1)      # the documented saturation
+
+
+def test_single_key_rows_with_a_large_norm_factor_get_no_score_gradient():
+    """Under the causal mask the first query sees one key: its softmax is 1 whatever q and k are, so dq of that
+    row is exactly zero.  With lambda just above 1 the two streams nearly cancel there, the norm factor is
+    large (rsqrt of a mean square near eps) and dX with it; dS = A (dP - delta) then cancels two large numbers,
+    which only comes out when delta is formed from the same rounded dX that the products read."""
+    from layers import MultiheadDiffAttnKernel
+
+    B, H, N, D = 2, 1, 37, 64
+    g = torch.Generator().manual_seed(5586)
+    mk = lambda d, s=1.0: (torch.randn(B, H, N, d, generator=g) * s).half()
+    q1, q2, k1, k2 = (mk(D, 2.0) for _ in range(4))
+    v, dy = mk(2 * D), mk(2 * D)
+    lam = torch.tensor([1.005], dtype=torch.float32)
+    leaves = [t.cuda().requires_grad_(True) for t in (q1, q2, k1, k2, v)]
+    lam_dev = lam.cuda().requires_grad_(True)
+    y = MultiheadDiffAttnKernel(*leaves, lambda_scale=lam_dev, lambda_init=0.8, rms_norm=True, causal=True)
+    y.backward(dy.cuda())
+    torch.cuda.synchronize()
+    ref = orc.forward_backward(q1, q2, k1, k2, v, lam, dy, 0.8, True, causal=True)
+    assert max_abs(y.detach(), ref[0]) <= Y_ATOL
+    for name, t, want in zip(("dq1", "dq2"), leaves[:2], ref[1:3]):
+        assert want[:, :, 0].abs().max().item() == 0.0                     # the oracle agrees: no gradient
+        first_row = t.grad[:, :, 0].float().abs().max().item()
+        assert first_row <= 1e-2 * want.abs().max().item(), (name, first_row)
+    for name, t, want in zip(("dk1", "dk2"), leaves[2:4], ref[3:5]):
+        assert rel_to_max(t.grad, want) <= GRAD_RTOL, name

@@ -79,22 +79,31 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) { dx[e] = (float)g8[e]; x[e] = (float)y8[e]; }
     }
-    float t2 = 0.f, tx = 0.f;
+    // The row sums delta are formed from dX as the other kernels will read it, rounded to 16 bits: dS = A (dP - delta)
+    // with dP = dX V^T cancels almost completely where a row attends to a single key, and a delta from the
+    // unrounded dX would leave the rounding error of dX times V behind, scaled by a norm factor that is large
+    // exactly in the rows where the two streams nearly cancel.  (The reference takes delta from the unrounded
+    // gradient, src/kernel.py:290-296, and dP from the rounded one, :374-375 and :419.)  d(lambda) has no such
+    // cancellation and takes the unrounded values.
+    float t2 = 0.f, t2r = 0.f, tx = 0.f;
     h8 d8;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      t2 += dx[e] * (float)u8[e];
-      tx += dx[e] * x[e];
       d8[e] = (half_t)dx[e];
+      const float dxr = (float)d8[e];
+      t2 += dx[e] * (float)u8[e];
+      t2r += dxr * (float)u8[e];
+      tx += dxr * x[e];
     }
 #pragma unroll
     for (int msk = LPR / 2; msk >= 1; msk >>= 1) {
       t2 += __shfl_xor(t2, msk, 64);
+      t2r += __shfl_xor(t2r, msk, 64);
       tx += __shfl_xor(tx, msk, 64);
     }
     *reinterpret_cast<h8*>(p.dx + off) = d8;
     if (sub == 0) {
-      const float delta2 = -lam * t2;
+      const float delta2 = -lam * t2r;
       p.stat[0 * rows + row] = -p.lse1[row] * kLog2e;
       p.stat[1 * rows + row] = -p.lse2[row] * kLog2e;
       const float delta1 = tx - delta2;
