@@ -56,54 +56,53 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(BwdParams p) {
       g8 = *reinterpret_cast<const h8*>(gdy + n * (size_t)p.sdy.n);
     }
     const h8 u8 = *reinterpret_cast<const h8*>(p.u2 + off);
-    float dx[8], x[8];
+    // dX of the row, and ix with X = ix * Y (the pre-norm row rebuilt from the saved output)
+    float dx[8], ix = 1.0f;
     if (RMS) {
       float gy = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) gy += (float)g8[e] * (float)y8[e];
+      for (int e = 0; e < 8; e += 2) gy = dot_pair(h2{g8[e], g8[e + 1]}, h2{y8[e], y8[e + 1]}, gy);
 #pragma unroll
       for (int msk = LPR / 2; msk >= 1; msk >>= 1) gy += __shfl_xor(gy, msk, 64);
       const float r = p.rinv[row];
       if (c != 0.f) {
-        const float a = c * r, b = r * gy / (c * DV), ix = 1.0f / (c * r);
+        const float a = c * r, b = r * gy / (c * DV);
+        ix = 1.0f / (c * r);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          dx[e] = a * (float)g8[e] - b * (float)y8[e];
-          x[e] = (float)y8[e] * ix;
-        }
+        for (int e = 0; e < 8; ++e) dx[e] = a * (float)g8[e] - b * (float)y8[e];
       } else {
+        ix = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { dx[e] = 0.f; x[e] = 0.f; }
+        for (int e = 0; e < 8; ++e) dx[e] = 0.f;
       }
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) { dx[e] = (float)g8[e]; x[e] = (float)y8[e]; }
+      for (int e = 0; e < 8; ++e) dx[e] = (float)g8[e];
     }
-    // The row sums delta are formed from dX as the other kernels will read it, rounded to 16 bits: dS = A (dP - delta)
+    // The row sums are formed from dX as the other kernels will read it, rounded to 16 bits: dS = A (dP - delta)
     // with dP = dX V^T cancels almost completely where a row attends to a single key, and a delta from the
     // unrounded dX would leave the rounding error of dX times V behind, scaled by a norm factor that is large
     // exactly in the rows where the two streams nearly cancel.  (The reference takes delta from the unrounded
-    // gradient, src/kernel.py:290-296, and dP from the rounded one, :374-375 and :419.)  d(lambda) has no such
-    // cancellation and takes the unrounded values.
-    float t2 = 0.f, t2r = 0.f, tx = 0.f;
+    // gradient, src/kernel.py:290-296, and dP from the rounded one, :374-375 and :419.)  The products of the
+    // 16-bit values are exact and summed in fp32.
+    float t2 = 0.f, ty = 0.f;
     h8 d8;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      d8[e] = (half_t)dx[e];
-      const float dxr = (float)d8[e];
-      t2 += dx[e] * (float)u8[e];
-      t2r += dxr * (float)u8[e];
-      tx += dxr * x[e];
+    for (int e = 0; e < 8; ++e) d8[e] = (half_t)dx[e];
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+      t2 = dot_pair(h2{d8[e], d8[e + 1]}, h2{u8[e], u8[e + 1]}, t2);
+      ty = dot_pair(h2{d8[e], d8[e + 1]}, h2{y8[e], y8[e + 1]}, ty);
     }
 #pragma unroll
     for (int msk = LPR / 2; msk >= 1; msk >>= 1) {
       t2 += __shfl_xor(t2, msk, 64);
-      t2r += __shfl_xor(t2r, msk, 64);
-      tx += __shfl_xor(tx, msk, 64);
+      ty += __shfl_xor(ty, msk, 64);
     }
+    const float tx = ty * ix;      // rowsum(dX * X)
     *reinterpret_cast<h8*>(p.dx + off) = d8;
     if (sub == 0) {
-      const float delta2 = -lam * t2r;
+      const float delta2 = -lam * t2;
       p.stat[0 * rows + row] = -p.lse1[row] * kLog2e;
       p.stat[1 * rows + row] = -p.lse2[row] * kLog2e;
       const float delta1 = tx - delta2;

@@ -74,6 +74,15 @@ __device__ __forceinline__ float add_pair(h2 x, float acc) {
 #endif
 }
 
+// acc + a[0]*b[0] + a[1]*b[1] in one instruction, the products of 16-bit values exact and summed in fp32
+__device__ __forceinline__ float dot_pair(h2 a, h2 b, float acc) {
+#ifdef DA_BF16
+  return __builtin_amdgcn_fdot2_f32_bf16(a, b, acc, false);
+#else
+  return __builtin_amdgcn_fdot2(a, b, acc, false);
+#endif
+}
+
 // MFMA with the B operand held in an accumulation register (AGPR) and the result in ordinary
 // VGPRs.  Used where B is a loop-invariant fragment: it then lives in the AGPR half of the register
 // file for the whole kernel, at no cost in VGPRs and without copies.  Being inline assembly, the
