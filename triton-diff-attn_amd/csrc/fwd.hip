@@ -30,6 +30,10 @@ struct FwdCfg {
   static constexpr int NW = 2 * BM / (32 * QS);    // waves per workgroup: half of them per softmax stream
   static constexpr int NT = NW * 64;
   static constexpr int OCC = (QS == 2 || D == 128) ? 1 : 2;   // waves per SIMD the register budget is sized for
+  // thread count the register budget is derived from: with fewer than 4 * OCC waves in a workgroup the
+  // occupancy attribute alone does not hold the allocator to 512 / OCC registers (the four-wave variant at
+  // D = 64 then took 336 and shuffled values between the two halves of the register file all through its loop)
+  static constexpr int REG_NT = (OCC * 256 > NT) ? OCC * 256 : NT;
   static constexpr int K_TILE = BN * D;            // halfs, one stream (swizzled, unpadded)
   static constexpr int V_TILE = BN * DV;
   static constexpr int K_BUF = 2 * K_TILE;         // K1 and K2 of one tile
@@ -59,7 +63,7 @@ constexpr float kRescaleThreshold = 8.0f;   // log2 units: probabilities stay be
 // src/kernel.py:4): a dropped probability still counts in its row's sum but not in P*V, and the
 // kept ones are scaled by 1/(1-p) -- in the epilogue, together with 1/l.
 template <int D, bool RMS, int MASK, bool DROP, bool SMALL = false>
-__global__ __launch_bounds__((FwdCfg<D, SMALL>::NT)) __attribute__((amdgpu_waves_per_eu(FwdCfg<D, SMALL>::OCC, FwdCfg<D, SMALL>::OCC)))
+__global__ __launch_bounds__((FwdCfg<D, SMALL>::REG_NT)) __attribute__((amdgpu_waves_per_eu(FwdCfg<D, SMALL>::OCC, FwdCfg<D, SMALL>::OCC)))
 void fwd_kernel(FwdParams p) {
   using C = FwdCfg<D, SMALL>;
   constexpr int DV = C::DV, BN = C::BN, NW = C::NW, BM = C::BM, QS = C::QS;
