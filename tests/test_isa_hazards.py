@@ -45,7 +45,7 @@ def assembly(tmp_path_factory):
     jobs = {}
     for key, src, variant in (("bwd_fp16", "bwd.hip", []), ("bwd_bf16", "bwd.hip", ["-DDA_BF16"]), ("fwd_fp16", "fwd.hip", [])):
         out = tmp / (key + ".s")
-        cmd = [build.HIPCC] + [f for f in build.FLAGS if f != "-fPIC"] + variant + ["--cuda-device-only", "-S", "-o", str(out),
+        cmd = [build.HIPCC] + [f for f in build.FLAGS if f != "-fPIC"] + build.SOURCE_FLAGS.get(src, []) + variant + ["--cuda-device-only", "-S", "-o", str(out),
                                                                               os.path.join(CSRC, src)]
         jobs[key] = (out, subprocess.Popen(cmd, stdout=subprocess.DEVNULL, stderr=subprocess.PIPE))
     texts = {}

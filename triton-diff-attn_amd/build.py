@@ -22,6 +22,12 @@ FLAGS = [
 ]
 # the kernel sources are compiled with per-kernel resource remarks, which check_resources() reads
 REMARKS = ["-Rpass-analysis=kernel-resource-usage"]
+# Flags of single sources.  A kernel sized for one wave per SIMD may use 512 registers, and for such a kernel the
+# compiler selects every MFMA in the form whose C and D operands are AGPRs, so each score that the VALU reads
+# next costs a copy (and each reference value a copy the other way): the D = 128 forward issued two such copies
+# per matrix product.  In the VGPR form its loop needs 268 registers and no copies (1.83 -> 1.75 ms at B2 H32
+# N4096).  Not for the backward source, whose dK/dV kernels place their operands by hand.
+SOURCE_FLAGS = {"fwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def check_resources(src, remarks):
@@ -55,7 +61,7 @@ def build(verbose=True):
     for src, extra, obj_name in units:
         obj = os.path.join(CSRC, obj_name)
         remarks = REMARKS if src in KERNEL_SOURCES else []
-        cmd = [HIPCC, *FLAGS, *remarks, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [HIPCC, *FLAGS, *SOURCE_FLAGS.get(src, []), *remarks, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
