@@ -18,18 +18,20 @@
 
 namespace DA_NS {
 
-// SMALL: 64 query rows per workgroup at D <= 64 as well, for problems whose 128-row blocks do not fill the chip.
+// SMALL: 64 query rows per workgroup (four waves), for problems whose 128-row blocks do not fill the chip and
+// for the D = 128 instantiations that do not fit the register budget of two waves per SIMD.
 template <int D, bool SMALL = false>
 struct FwdCfg {
   static constexpr int DV = 2 * D;
   static constexpr int BN = (D <= 64) ? 64 : 32;   // keys per tile
   static constexpr int QS = 1;                     // 32-row query blocks per wave
-  // query rows per workgroup; the output accumulators of a D = 128 wave need more than 256
-  // registers, so those workgroups have four waves at one wave per SIMD
-  static constexpr int BM = (D == 128 || SMALL) ? 64 : 128;
+  // query rows per workgroup
+  static constexpr int BM = SMALL ? 64 : 128;
   static constexpr int NW = 2 * BM / (32 * QS);    // waves per workgroup: half of them per softmax stream
   static constexpr int NT = NW * 64;
-  static constexpr int OCC = (QS == 2 || D == 128) ? 1 : 2;   // waves per SIMD the register budget is sized for
+  // waves per SIMD the register budget is sized for: two, except in the four-wave D = 128 workgroups, whose
+  // masked and dropout instantiations need more than 256 registers
+  static constexpr int OCC = (D == 128 && SMALL) ? 1 : 2;
   // thread count the register budget is derived from: with fewer than 4 * OCC waves in a workgroup the
   // occupancy attribute alone does not hold the allocator to 512 / OCC registers (the four-wave variant at
   // D = 64 then took 336 and shuffled values between the two halves of the register file all through its loop)
@@ -50,8 +52,9 @@ struct FwdCfg {
   // halfs needed by the epilogue: per pair of waves (stream 1, stream 2 of the same 32 rows) an fp32 exchange
   // block of 32 x DV values, which the stream-1 wave reuses for its staged rows, and the staging block
   // (32 rows of DV + 8 halfs) of the stream-2 wave
-  static constexpr int XCH_BLOCK = 64 * DV;
-  static constexpr int XCHG = (NW / 2) * (XCH_BLOCK + 32 * (DV + 8));
+  // (a block holds the exchange, and after it has been read the staged rows of both waves of the pair)
+  static constexpr int XCH_BLOCK = (64 * DV > 2 * 32 * (DV + 8)) ? 64 * DV : 2 * 32 * (DV + 8);
+  static constexpr int XCHG = (NW / 2) * XCH_BLOCK;
   static constexpr int SMEM = (TILES > XCHG) ? TILES : XCHG;
 };
 
@@ -480,11 +483,11 @@ void fwd_kernel(FwdParams p) {
   // (src/kernel.py:191-194), so that rows in which the two streams nearly cancel (lambda near 1, similar
   // attention maps) do not see the rounding error of one stream amplified by the norm.  The two waves
   // hold a row's values in the same lanes and registers, so the exchange is lane to lane.
+  // Each pair of waves has one block of tile memory: first it carries the fp32 exchange, then, once the
+  // workgroup has met behind the combine, the staged rows of the two waves side by side.
   constexpr int SROW = DV + 8;
   float* const xch = reinterpret_cast<float*>(smem + (size_t)qw * C::XCH_BLOCK);
-  // stream 1 stages its rows in its pair's exchange block, which only this wave reads, after reading it
-  half_t* const stg_own = st ? smem + (size_t)(NW / 2) * C::XCH_BLOCK + (size_t)qw * 32 * SROW
-                             : smem + (size_t)qw * C::XCH_BLOCK;
+  half_t* const stg_own = smem + (size_t)qw * C::XCH_BLOCK + (st ? 32 * SROW : 0);
   auto stage_rows = [&](int qs, const f16v (&val)[NOT], float scale) {
 #pragma unroll
     for (int tt = 0; tt < NOT; ++tt)
@@ -520,7 +523,6 @@ void fwd_kernel(FwdParams p) {
     if (g == 0 && lse) lse[row] = (m[0] + __builtin_log2f(lsum)) * kLn2;
   }
   if (st == 1) {
-    stage_rows(0, o[0], inv);
 #pragma unroll
     for (int tt = 0; tt < NOT; ++tt)
 #pragma unroll
@@ -532,11 +534,9 @@ void fwd_kernel(FwdParams p) {
       }
   }
   __syncthreads();
-  if (st == 1) {
-    if (p.u2) store_rows(p.u2 + wave_row0 * DV, DV, 32);
-  } else {
-    const float lam = da_abi::lambda_of_unit(p, bh);
-    float ss = 0.f;
+  const float lam = da_abi::lambda_of_unit(p, bh);
+  float ss = 0.f;
+  if (st == 0) {
 #pragma unroll
     for (int tt = 0; tt < NOT; ++tt)
 #pragma unroll
@@ -549,6 +549,13 @@ void fwd_kernel(FwdParams p) {
           ss += x * x;
         }
       }
+  }
+  __syncthreads();      // the exchange has been read: the blocks may take the staged rows
+  if (st == 1) {
+    stage_rows(0, o[0], inv);
+    __builtin_amdgcn_wave_barrier();   // the rows are read back by other lanes of this wave only
+    if (p.u2) store_rows(p.u2 + wave_row0 * DV, DV, 32);
+  } else {
     float scale = 1.0f;
     if (RMS) {
       ss = pair_sum(ss);
@@ -563,44 +570,55 @@ void fwd_kernel(FwdParams p) {
   }
 }
 
-template <int D, bool RMS, bool DROP>
-static void launch_fwd_c(const FwdParams& p, dim3 grid, dim3 block, hipStream_t stream) {
+template <int D, bool RMS, bool DROP, bool SMALL>
+static void launch_fwd_c(const FwdParams& p, hipStream_t stream) {
+  using C = FwdCfg<D, SMALL>;
+  const dim3 grid(p.BH * (p.N / C::BM)), block(C::NT);
   if (p.causal)
-    hipLaunchKernelGGL((fwd_kernel<D, RMS, 1, DROP>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, 1, DROP, SMALL>), grid, block, 0, stream, p);
   else if (p.n_keys < p.N)
-    hipLaunchKernelGGL((fwd_kernel<D, RMS, 2, DROP>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, 2, DROP, SMALL>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL((fwd_kernel<D, RMS, 0, DROP>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((fwd_kernel<D, RMS, 0, DROP, SMALL>), grid, block, 0, stream, p);
 }
 
 template <int D>
 static hipError_t launch_fwd_t(const FwdParams& p, hipStream_t stream) {
-  dim3 grid(p.BH * (p.N / FwdCfg<D>::BM)), block(FwdCfg<D>::NT);
   const bool drop = p.drop.threshold != 0;
+  const bool plain = !p.causal && !drop && p.n_keys == p.N;
   // Shape-aware launch geometry (the reference autotunes its tiles per (N, D, Dv), src/kernel.py:12-19): a problem
-  // whose 128-row blocks do not fill the chip once runs in twice as many 64-row workgroups.  A pure function of
-  // (B*H, N, D) and the options: no tuning state.  Only the plain instantiations have the small variant.
+  // whose 128-row blocks do not fill the chip once runs in twice as many 64-row, four-wave workgroups.  A pure
+  // function of (B*H, N, D) and the options: no tuning state.  At D <= 64 only the plain instantiation has the
+  // small variant.  At D = 128 it is the other way round: only the plain instantiation fits the 256 registers of
+  // the 128-row workgroup (two waves per SIMD); with a mask or dropout the kernel runs in 64-row workgroups at one
+  // wave per SIMD.
   constexpr int kNumCU = 256;
-  if constexpr (D != 128) {
-    if (!p.causal && !drop && p.n_keys == p.N && (long long)p.BH * (p.N / 128) < kNumCU) {
+  const bool small_grid = (long long)p.BH * (p.N / 128) < kNumCU;
+  if constexpr (D == 128) {
+    if (!plain || small_grid) {
+      if (p.rms_norm) { if (drop) launch_fwd_c<D, true, true, true>(p, stream); else launch_fwd_c<D, true, false, true>(p, stream); }
+      else            { if (drop) launch_fwd_c<D, false, true, true>(p, stream); else launch_fwd_c<D, false, false, true>(p, stream); }
+    } else {
+      const dim3 grid(p.BH * (p.N / FwdCfg<D>::BM)), block(FwdCfg<D>::NT);
+      if (p.rms_norm) hipLaunchKernelGGL((fwd_kernel<D, true, 0, false, false>), grid, block, 0, stream, p);
+      else            hipLaunchKernelGGL((fwd_kernel<D, false, 0, false, false>), grid, block, 0, stream, p);
+    }
+    return hipGetLastError();
+  } else {
+    if (plain && small_grid) {
       const dim3 sgrid(p.BH * (p.N / FwdCfg<D, true>::BM)), sblock(FwdCfg<D, true>::NT);
       if (p.rms_norm) hipLaunchKernelGGL((fwd_kernel<D, true, 0, false, true>), sgrid, sblock, 0, stream, p);
       else            hipLaunchKernelGGL((fwd_kernel<D, false, 0, false, true>), sgrid, sblock, 0, stream, p);
       return hipGetLastError();
     }
+    if (p.rms_norm) { if (drop) launch_fwd_c<D, true, true, false>(p, stream); else launch_fwd_c<D, true, false, false>(p, stream); }
+    else            { if (drop) launch_fwd_c<D, false, true, false>(p, stream); else launch_fwd_c<D, false, false, false>(p, stream); }
+    return hipGetLastError();
   }
-  if (p.rms_norm) {
-    if (drop) launch_fwd_c<D, true, true>(p, grid, block, stream);
-    else      launch_fwd_c<D, true, false>(p, grid, block, stream);
-  } else {
-    if (drop) launch_fwd_c<D, false, true>(p, grid, block, stream);
-    else      launch_fwd_c<D, false, false>(p, grid, block, stream);
-  }
-  return hipGetLastError();
 }
 
 // Tile-size choice per head dimension (replaces the reference's run-time autotuner,
-// src/kernel.py:12-19): 128 query rows per workgroup and 64 keys per step for D <= 64; 64 rows and 32 keys for D = 128.
+// src/kernel.py:12-19): 128 query rows per workgroup; 64 keys per step for D <= 64, 32 for D = 128.
 hipError_t launch_fwd(const FwdParams& p, int D, hipStream_t stream) {
   switch (D) {
     case 32:  return launch_fwd_t<32>(p, stream);
