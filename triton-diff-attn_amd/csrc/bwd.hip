@@ -749,6 +749,9 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   constexpr bool TAIL = (MASK != 0);
   constexpr int DV = C::DV, NW = C::NW, BM = C::BM, BN = C::BN;
   constexpr int NKS = D / 16, NKV = DV / 16, NDT = D / 32;
+#ifndef DQ_ASM_SCORES
+#define DQ_ASM_SCORES (D == 128 && !DROP)
+#endif
 
   __shared__ __attribute__((aligned(16))) half_t smem[C::NBUF * C::STAGE];
   static_assert(sizeof(smem) >= 256 * sizeof(float), "the hosted reduction uses the tile memory");
@@ -856,8 +859,22 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   // used.  It does not see the asynchronous tile copies, so its wait for "the newest loads" would in fact be a
   // wait for every tile copy in flight, in every iteration.  Touching the registers here puts that wait in front
   // of the loop, where the first tiles are waited for anyway.
+  // At D = 128 the kernel runs one wave per SIMD, and for a kernel with that register budget the compiler selects
+  // every MFMA with its C and D operands in AGPRs: right for the dQ accumulators, but each recomputed score
+  // and dP value then costs a copy back for the element-wise work (a quarter of the loop's VALU instructions).
+  // There the three score products are issued as assembly with their results in VGPRs and the resident
+  // Q1, Q2 and dX rows, which are only ever B operands, in AGPRs.  (Not in the dropout instantiations, whose
+  // mask arithmetic makes the compiler move operands about: see bwd_dkdv_kernel.)
+  constexpr bool kAsmScores = DQ_ASM_SCORES;
+  if constexpr (kAsmScores) {
 #pragma unroll
-  for (int kv = 0; kv < NKV; ++kv) asm volatile("" : "+v"(xf[kv]));
+    for (int ks = 0; ks < NKS; ++ks) { keep_in_agpr(qf1[ks]); keep_in_agpr(qf2[ks]); }
+#pragma unroll
+    for (int kv = 0; kv < NKV; ++kv) keep_in_agpr(xf[kv]);
+  } else {
+#pragma unroll
+    for (int kv = 0; kv < NKV; ++kv) asm volatile("" : "+v"(xf[kv]));
+  }
   float nl1 = nl1_ld, nl2 = nl2_ld, de1 = de1_ld, de2 = de2_ld;
   asm volatile("" : "+v"(nl1), "+v"(nl2), "+v"(de1), "+v"(de2));
   if (C::PAIR) wait_async_tiles();                  // tiles 0 and 1 are read before the next barrier
@@ -891,10 +908,10 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   // Where registers allow, a row statistic that is added to every element of a product is the product's
   // initial accumulator value instead: sixteen registers that hold it, for sixteen additions less per sub-tile.
 #ifndef DQ_FOLD_DP
-#define DQ_FOLD_DP (!DROP && (D == 32 || (D == 64 && MASK == 0)))
+#define DQ_FOLD_DP (!DROP && (D == 32 || (D == 64 && MASK == 0) || (D == 128 && MASK == 0)))
 #endif
 #ifndef DQ_FOLD_S
-#define DQ_FOLD_S (D == 32)
+#define DQ_FOLD_S (D == 32 || (D == 128 && MASK == 0 && !DROP))
 #endif
   constexpr bool kFoldDP = DQ_FOLD_DP;     // dP starts from -delta1 (not with dropout, which masks dP first)
   constexpr bool kFoldS = DQ_FOLD_S;       // S1, S2 start from the negated logsumexp
@@ -927,13 +944,32 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
 #pragma unroll
       for (int kv = 0; kv < NKV; ++kv) av[kv] = lds_read_at<h8>(vfr[kv], VCUR + ksub * 32 * DV * 2);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kAsmScores) {
+        if constexpr (kFoldS) {
+          s1 = mfma32_bagpr_from(ak1[0], qf1[0], nl1v);
+          s2 = mfma32_bagpr_from(ak2[0], qf2[0], nl2v);
+        } else {
+          s1 = mfma32_bagpr_first(ak1[0], qf1[0]);
+          s2 = mfma32_bagpr_first(ak2[0], qf2[0]);
+        }
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        s1 = mfma32(ak1[ks], qf1[ks], s1);
-        s2 = mfma32(ak2[ks], qf2[ks], s2);
+        for (int ks = 1; ks < NKS; ++ks) {
+          s1 = mfma32_bagpr(ak1[ks], qf1[ks], s1);
+          s2 = mfma32_bagpr(ak2[ks], qf2[ks], s2);
+        }
+        dp = kFoldDP ? mfma32_bagpr_from(av[0], xf[0], de1v) : mfma32_bagpr_first(av[0], xf[0]);
+#pragma unroll
+        for (int kv = 1; kv < NKV; ++kv) dp = mfma32_bagpr(av[kv], xf[kv], dp);
+        mfma_results_ready(s1, s2, dp);      // the compiler does not know these are matrix instructions
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+          s1 = mfma32(ak1[ks], qf1[ks], s1);
+          s2 = mfma32(ak2[ks], qf2[ks], s2);
+        }
+#pragma unroll
+        for (int kv = 0; kv < NKV; ++kv) dp = mfma32(av[kv], xf[kv], dp);
       }
-#pragma unroll
-      for (int kv = 0; kv < NKV; ++kv) dp = mfma32(av[kv], xf[kv], dp);
       if (ksub == 0) copy_v(tn, v_buf(BNXT), v_begin, v_mid);
       // with a barrier every second tile all of a tile's copies go out early: they have to land by the next barrier
       if (ksub == (C::PAIR ? 0 : BN / 32 - 1)) copy_v(tn, v_buf(BNXT), v_mid, v_end);

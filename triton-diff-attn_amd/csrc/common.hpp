@@ -92,6 +92,18 @@ __device__ __forceinline__ f16v mfma32_bagpr(h8 a, h8 b, f16v c) {
   asm volatile(DA_MFMA_32x32x16 " %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
   return c;
 }
+// The same, starting a sum: C is the constant zero.
+__device__ __forceinline__ f16v mfma32_bagpr_first(h8 a, h8 b) {
+  f16v c;
+  asm volatile(DA_MFMA_32x32x16 " %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+  return c;
+}
+// The same, starting from a given accumulator value that stays as it is.
+__device__ __forceinline__ f16v mfma32_bagpr_from(h8 a, h8 b, const f16v& c0) {
+  f16v c;
+  asm volatile(DA_MFMA_32x32x16 " %0, %1, %2, %3" : "=&v"(c) : "v"(a), "a"(b), "v"(c0));
+  return c;
+}
 // Moves a fragment into AGPRs for good: after this the value is defined by an (empty) asm statement
 // with an AGPR output, so the compiler has no VGPR original to copy from in front of a later use.
 // A v_accvgpr_write directly in front of an inline-asm MFMA that reads the AGPR is a hazard the
