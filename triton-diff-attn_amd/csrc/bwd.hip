@@ -752,6 +752,10 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
 #ifndef DQ_ASM_SCORES
 #define DQ_ASM_SCORES (D == 128 && !DROP)
 #endif
+#ifndef DQ_PIPE
+#define DQ_PIPE (D == 128 && !DROP)
+#endif
+  constexpr bool kPipe = DQ_PIPE;     // the software-pipelined loop of the one-wave-per-SIMD kernel, below
 
   __shared__ __attribute__((aligned(16))) half_t smem[C::NBUF * C::STAGE];
   static_assert(sizeof(smem) >= 256 * sizeof(float), "the hosted reduction uses the tile memory");
@@ -855,6 +859,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   const int b0 = head_half ? 2 : 0;
   fetch_all(0, b0);
   fetch_all((n_tiles > 1) ? 1 : 0, b0 + 1);
+  if constexpr (kPipe) fetch_all((n_tiles > 2) ? 2 : n_tiles - 1, (b0 + 2) % C::NBUF);   // it fetches three tiles ahead
   // dX and the row statistics are first used inside the loop, and the compiler waits for a load where it is first
   // used.  It does not see the asynchronous tile copies, so its wait for "the newest loads" would in fact be a
   // wait for every tile copy in flight, in every iteration.  Touching the registers here puts that wait in front
@@ -877,7 +882,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   }
   float nl1 = nl1_ld, nl2 = nl2_ld, de1 = de1_ld, de2 = de2_ld;
   asm volatile("" : "+v"(nl1), "+v"(nl2), "+v"(de1), "+v"(de2));
-  if (C::PAIR) wait_async_tiles();                  // tiles 0 and 1 are read before the next barrier
+  if (C::PAIR || kPipe) wait_async_tiles();         // tiles 0 and 1 are read before the next barrier
   else wait_async_tiles_except(loads_per_iter);     // tile 0 has landed, tile 1 may still be in flight
   __syncthreads();
 
@@ -908,10 +913,10 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   // Where registers allow, a row statistic that is added to every element of a product is the product's
   // initial accumulator value instead: sixteen registers that hold it, for sixteen additions less per sub-tile.
 #ifndef DQ_FOLD_DP
-#define DQ_FOLD_DP (!DROP && (D == 32 || (D == 64 && MASK == 0) || (D == 128 && MASK == 0)))
+#define DQ_FOLD_DP (!DROP && (D == 32 || (D == 64 && MASK == 0)))
 #endif
 #ifndef DQ_FOLD_S
-#define DQ_FOLD_S (D == 32 || (D == 128 && MASK == 0 && !DROP))
+#define DQ_FOLD_S (D == 32)
 #endif
   constexpr bool kFoldDP = DQ_FOLD_DP;     // dP starts from -delta1 (not with dropout, which masks dP first)
   constexpr bool kFoldS = DQ_FOLD_S;       // S1, S2 start from the negated logsumexp
@@ -921,6 +926,140 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
   if constexpr (kFoldDP) asm volatile("" : "+v"(de1v));
   if constexpr (kFoldS) asm volatile("" : "+v"(nl1v), "+v"(nl2v));
 
+  if constexpr (kPipe) {
+    // One wave per SIMD has nobody to run its element-wise work under, so the loop is pipelined inside the wave,
+    // as in the dK/dV kernel: while the element-wise work of tile t runs on the VALU, row by row, the score
+    // products of tile t+1 (assembly, results in VGPRs) run on the matrix unit, two per row; the dQ products
+    // of tile t follow.  Tiles are 32 keys (one sub-tile) and are fetched three iterations ahead; the workgroup
+    // meets once per tile.
+    static_assert(kAsmScores && BN == 32 && !kFoldDP && !kFoldS, "the pipelined loop");
+    struct Scores { f16v s1, s2, dp; };
+    constexpr int NPROD = 2 * NKS + NKV;              // score products per tile: S1 and S2 alternating, then dP
+    // A fragment of product k of the tile in the buffer at byte offsets (KOFF, VOFF)
+    auto prod_frag = [&](auto koff_tag, auto voff_tag, int k) -> h8 {
+      constexpr int KOFF = decltype(koff_tag)::value, VOFF = decltype(voff_tag)::value;
+      if (k < 2 * NKS) return lds_read_at<h8>(kfr[k / 2], KOFF + (k & 1) * C::K_TILE * 2);
+      return lds_read_at<h8>(vfr[k - 2 * NKS], VOFF);
+    };
+    auto prod_mfma = [&](int k, h8 a, Scores& s) {
+      if (k < 2 * NKS) {
+        const int ks = k / 2;
+        if (k & 1) s.s2 = ks ? mfma32_bagpr(a, qf2[ks], s.s2) : mfma32_bagpr_first(a, qf2[0]);
+        else       s.s1 = ks ? mfma32_bagpr(a, qf1[ks], s.s1) : mfma32_bagpr_first(a, qf1[0]);
+      } else {
+        const int kv = k - 2 * NKS;
+        s.dp = kv ? mfma32_bagpr(a, xf[kv], s.dp) : mfma32_bagpr_first(a, xf[0]);
+      }
+    };
+    constexpr int DEPTH = 4;                          // A fragments requested ahead of their product
+    Scores sa, sb;
+    {
+      // scores of tile 0, nothing to run them under
+      h8 a[NPROD];
+      if (head_half) {
+#pragma unroll
+        for (int k = 0; k < NPROD; ++k)
+          a[k] = prod_frag(std::integral_constant<int, 2 * C::KBUF_BYTES>{}, std::integral_constant<int, 2 * C::VBUF_BYTES>{}, k);
+      } else {
+#pragma unroll
+        for (int k = 0; k < NPROD; ++k) a[k] = prod_frag(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, k);
+      }
+#pragma unroll
+      for (int k = 0; k < NPROD; ++k) prod_mfma(k, a[k], sa);
+      mfma_results_ready(sa.s1, sa.s2, sa.dp);
+    }
+
+    auto iteration = [&](int t, auto pos_tag, Scores& cur, Scores& nxt) {
+      constexpr int POS = decltype(pos_tag)::value;
+      constexpr int KCUR = POS * C::KBUF_BYTES;
+      constexpr int PNXT = (POS + 1) % C::NBUF, BFAR = (POS + 3) % C::NBUF;
+      constexpr std::integral_constant<int, PNXT * C::KBUF_BYTES> knext{};
+      constexpr std::integral_constant<int, PNXT * C::VBUF_BYTES> vnext{};
+      const int tf = (t + 3 < n_tiles) ? t + 3 : n_tiles - 1;   // past the end: harmless re-reads
+      copy_k(gk1, tf, k_buf(BFAR));
+      if constexpr (CAUSAL) {
+        // only the last tiles of a wave's loop reach past its first row: mask key > query there
+        const int wrow0 = qt * BM + wave * 32;
+        const int kbase = t * BN;
+        if (kbase + 31 > wrow0) {
+          const int rel = wrow0 + j - kbase - 4 * g;     // query index minus the key index of register 0
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (8 * (r / 4) + (r % 4) > rel) { cur.s1[r] = -INFINITY; cur.s2[r] = -INFINITY; }
+        }
+      }
+      if constexpr (PADDED) {
+        const int kbase = t * BN;
+        if (kbase + 32 > p.n_keys) {
+          const int rel = p.n_keys - 1 - kbase - 4 * g;   // last real key minus the key index of register 0
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (8 * (r / 4) + (r % 4) > rel) { cur.s1[r] = -INFINITY; cur.s2[r] = -INFINITY; }
+        }
+      }
+      // the transposed K fragments of this tile's dQ products are requested here and arrive under the loop below
+      h8 tk1[2][NDT], tk2[2][NDT];
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int tt = 0; tt < NDT; ++tt) {
+          const int off = KCUR + 16 * kk * D * 2;
+          tk1[kk][tt] = join(lds_read_tr_at(ktr[tt][0], off), lds_read_tr_at(ktr[tt][1], off));
+          tk2[kk][tt] = join(lds_read_tr_at(ktr[tt][0], off + C::K_TILE * 2), lds_read_tr_at(ktr[tt][1], off + C::K_TILE * 2));
+        }
+      h8 a[NPROD];
+#pragma unroll
+      for (int k = 0; k < DEPTH; ++k) a[k] = prod_frag(knext, vnext, k);
+      h8 b1[2], b2[2];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int k = 0; k < NPROD; ++k) {
+        if (k + DEPTH < NPROD) a[k + DEPTH] = prod_frag(knext, vnext, k + DEPTH);
+        // the far tile's copies are spread over the products
+        if (k == NPROD / 4) copy_k(gk2, tf, k_buf(BFAR) + C::K_TILE);
+        if (k == NPROD / 2) copy_v(tf, v_buf(BFAR), v_begin, v_mid);
+        if (k == 3 * NPROD / 4) copy_v(tf, v_buf(BFAR), v_mid, v_end);
+        prod_mfma(k, a[k], nxt);
+        // element-wise rows of this tile, spread evenly over the products
+        const int r0 = 16 * k / NPROD, r1 = 16 * (k + 1) / NPROD;
+#pragma unroll
+        for (int r = r0; r < r1; ++r) {
+          const float p1 = fast_exp2(cur.s1[r] + nl1);
+          const float p2 = fast_exp2(cur.s2[r] + nl2);
+          // in fp32 up to the rounding of dS itself (see the loop of the other head dims)
+          const float dpc = cur.dp[r] + de1;
+          b1[r / 8][r % 8] = (half_t)(p1 * dpc);
+          b2[r / 8][r % 8] = (half_t)(p2 * __builtin_fmaf(-lam, dpc, de2));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mfma_results_ready(nxt.s1, nxt.s2, nxt.dp);     // the next iteration's VALU reads them
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int tt = 0; tt < NDT; ++tt) {
+          dq1[tt] = mfma32(tk1[kk][tt], b1[kk], dq1[tt]);
+          dq2[tt] = mfma32(tk2[kk][tt], b2[kk], dq2[tt]);
+        }
+      // the next iteration reads tiles t+1 and t+2: only this iteration's loads (tile t+3) may remain in flight
+      wait_async_tiles_except(loads_per_iter);
+      __syncthreads();
+    };
+
+    int t = 0;
+    if (head_half) {
+      iteration(0, std::integral_constant<int, 2>{}, sa, sb);
+      iteration(1, std::integral_constant<int, 3>{}, sb, sa);
+      t = 2;
+    }
+#pragma nounroll
+    for (; t < n_tiles; t += 4) {
+      iteration(t, std::integral_constant<int, 0>{}, sa, sb);
+      iteration(t + 1, std::integral_constant<int, 1>{}, sb, sa);
+      iteration(t + 2, std::integral_constant<int, 2>{}, sa, sb);
+      iteration(t + 3, std::integral_constant<int, 3>{}, sb, sa);
+    }
+  } else {
   // One iteration: tile t, in the buffer at ring position POS; tile t+2 is requested into the buffer two
   // positions on, which held a tile that every wave has finished reading.
   auto iteration = [&](int t, auto pos_tag) {
@@ -1081,6 +1220,7 @@ __global__ __launch_bounds__((DqCfg<D, NWAVES>::REG_NT)) __attribute__((amdgpu_w
     iteration(t + 1, std::integral_constant<int, 1>{});
     iteration(t + 2, std::integral_constant<int, 2>{});
     iteration(t + 3, std::integral_constant<int, 3>{});
+  }
   }
   wait_async_tiles();
   __syncthreads();      // the tile memory is reused below; other waves may still have been reading it
